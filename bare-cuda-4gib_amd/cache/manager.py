@@ -72,10 +72,39 @@ class View:
 PagedView = StateView = View     # (the two kinds of view were classes of their own once)
 
 
+class BundleView:
+    """The view of a stream whose spec names members: one attribute per member, that member's view."""
+
+    def __init__(self, members: Dict[str, Any]):
+        self.members = dict(members)
+        self.group = None
+
+    def __getattr__(self, name: str):
+        try:
+            return self.__dict__["members"][name]
+        except KeyError:
+            raise AttributeError(f"this cache stream has no member '{name}' (it has {sorted(self.__dict__.get('members', {}))})") from None
+
+    @property
+    def paged(self) -> bool:
+        return False
+
+
+def flatten_specs(specs: Iterable[Any]) -> List[Any]:
+    """The specs with every bundle replaced by its members."""
+    out = []
+    for spec in specs:
+        if spec is not None and hasattr(spec, "members"):
+            out.extend(flatten_specs(m for _, m in spec.members))
+        else:
+            out.append(spec)
+    return out
+
+
 def bytes_per_page(specs: Iterable[Any], page_tokens: int, dtype: torch.dtype) -> int:
     """Device bytes that one page index stands for, over all streams that keep something per token."""
     total = 0
-    for spec in specs:
+    for spec in flatten_specs(specs):
         if spec is not None and getattr(spec, "per_token", False):
             for entry in spec.page_tensors(page_tokens).values():
                 shape, dt = _shape_and_dtype(entry, dtype)
@@ -132,34 +161,12 @@ class CacheManager:
         self.poison = poison
         self.specs = dict(streams)
         self.groups: Dict[Hashable, _Group] = {}
-        self._views: Dict[Hashable, Any] = {}
+        self._views: Dict[Hashable, Any] = {}          # what a schedule entry's layer is handed, by stream
+        self._leaves: Dict[Hashable, View] = {}        # every view that holds tensors (a bundle's members: (stream, name))
         for sid, spec in self.specs.items():
-            if spec is None:
-                continue
-            if getattr(spec, "per_token", None) is True and hasattr(spec, "page_tensors"):
-                window = int(getattr(spec, "window", 0))
-                key, first_kept, keeps_all = _retention(spec)
-                group = self.groups.get(key)
-                if group is None:
-                    group = self.groups[key] = _Group(window, num_pages, first_kept, keeps_all)
-                group.streams.append(sid)
-                tensors = {}
-                for name, entry in spec.page_tensors(page_tokens).items():
-                    shape, dt = _shape_and_dtype(entry, dtype)
-                    t = torch.empty((num_pages + 1, *shape), dtype=dt, device=self.device)   # (+ the scratch page)
-                    if poison and t.is_floating_point():
-                        t.fill_(float("nan"))
-                    tensors[name] = t
-                self._views[sid] = View(tensors, group=key, page_tokens=page_tokens, window=window)
-            elif getattr(spec, "per_token", None) is False and hasattr(spec, "slot_tensors"):
-                tensors = {}
-                for name, entry in spec.slot_tensors().items():
-                    shape, dt = _shape_and_dtype(entry, dtype)
-                    tensors[name] = torch.zeros((max_requests + 1, *shape), dtype=dt, device=self.device)  # (+ the scratch slot)
-                self._views[sid] = View(tensors)
-            else:
-                raise EngineError(f"cache: stream {sid!r} has a spec that says neither what it keeps per token "
-                                  f"(per_token = True, page_tensors) nor per request (per_token = False, slot_tensors): {spec!r}")
+            view = self._make_view(sid, spec, num_pages)
+            if view is not None:
+                self._views[sid] = view
         self._requests: Dict[Hashable, _Request] = {}
         self._peaks: Dict[Tuple[int, int], Dict[Hashable, int]] = {}
         self._free_slots: List[int] = list(range(max_requests - 1, -1, -1))
@@ -176,6 +183,41 @@ class CacheManager:
             g: np.full((max_requests + 1, self.max_pages_per_request), -1, dtype=np.int32) for g in self.groups}
         for t in self.tables_by_slot.values():
             t[self.scratch_slot, 0] = self.scratch_page
+
+    def _make_view(self, sid: Hashable, spec: Any, num_pages: int):
+        """Allocates what the spec names and returns the stream's view (None for no spec)."""
+        dtype, page_tokens = self.dtype, self.page_tokens
+        if spec is None:
+            return None
+        if hasattr(spec, "members"):
+            made = {name: self._make_view((sid, name), member, num_pages) for name, member in spec.members}
+            return BundleView(made)
+        if getattr(spec, "per_token", None) is True and hasattr(spec, "page_tensors"):
+            window = int(getattr(spec, "window", 0))
+            key, first_kept, keeps_all = _retention(spec)
+            group = self.groups.get(key)
+            if group is None:
+                group = self.groups[key] = _Group(window, num_pages, first_kept, keeps_all)
+            group.streams.append(sid)
+            tensors = {}
+            for name, entry in spec.page_tensors(page_tokens).items():
+                shape, dt = _shape_and_dtype(entry, dtype)
+                t = torch.empty((num_pages + 1, *shape), dtype=dt, device=self.device)   # (+ the scratch page)
+                if self.poison and t.is_floating_point():
+                    t.fill_(float("nan"))
+                tensors[name] = t
+            view = View(tensors, group=key, page_tokens=page_tokens, window=window)
+        elif getattr(spec, "per_token", None) is False and hasattr(spec, "slot_tensors"):
+            tensors = {}
+            for name, entry in spec.slot_tensors().items():
+                shape, dt = _shape_and_dtype(entry, dtype)
+                tensors[name] = torch.zeros((self.max_requests + 1, *shape), dtype=dt, device=self.device)  # (+ the scratch slot)
+            view = View(tensors)
+        else:
+            raise EngineError(f"cache: stream {sid!r} has a spec that says neither what it keeps per token "
+                              f"(per_token = True, page_tensors) nor per request (per_token = False, slot_tensors): {spec!r}")
+        self._leaves[sid] = view
+        return view
 
     # ---- requests ---------------------------------------------------------
     def has(self, request: Hashable) -> bool:
@@ -197,7 +239,7 @@ class CacheManager:
         slot = self._free_slots.pop()
         self._requests[request] = _Request(slot, self.groups)
         self.lengths_by_slot[slot] = 0
-        for view in self._views.values():
+        for view in self._leaves.values():
             if not view.paged:
                 for t in view.tensors.values():
                     t[slot].zero_()
@@ -309,7 +351,7 @@ class CacheManager:
             raise EngineError(f"cache: page {page} of group {group} was freed twice or never held")
         if self.poison:
             for sid in self.groups[group].streams:
-                for t in self._views[sid].tensors.values():
+                for t in self._leaves[sid].tensors.values():
                     if t.is_floating_point():
                         t[page].fill_(float("nan"))
 
@@ -324,6 +366,18 @@ class CacheManager:
         self.lengths_by_slot[r.slot] = 0
         self._free_slots.append(r.slot)
         del self._requests[request]
+
+    def save_slots(self, slots: Sequence[int]):
+        """What the per-request tensors hold for these slots, to be put back with :meth:`restore_slots`: for whoever
+        has to run a step twice (once to warm up, once for good) without the state moving twice."""
+        index = torch.as_tensor(sorted(set(int(s) for s in slots)), dtype=torch.long, device=self.device)
+        return index, [(t, t[index].clone()) for view in self._leaves.values() if not view.paged
+                       for t in view.tensors.values() if t.numel()]
+
+    def restore_slots(self, saved) -> None:
+        index, kept = saved
+        for t, rows in kept:
+            t[index] = rows
 
     def peak_pages(self, total_tokens: int, portion: int) -> Dict[Hashable, int]:
         """group -> the most pages one request holds at a time while ``total_tokens`` tokens are fed
@@ -373,4 +427,4 @@ class CacheManager:
             g.pool.shuffle_free_list(seed + i)
 
     def storage_bytes(self) -> int:
-        return sum(t.numel() * t.element_size() for view in self._views.values() for t in view.tensors.values())
+        return sum(t.numel() * t.element_size() for view in self._leaves.values() for t in view.tensors.values())

@@ -16,6 +16,10 @@ per request ``per_token = False``.  ``slot_tensors()`` names the tensors of ONE 
             (name -> (shape, dtype name)); the manager allocates ``[max_requests, *shape]`` of each and
             zeroes a slot when a request is admitted to it.
 
+several     ``members`` names further specs (:class:`Bundle`): a layer that keeps more than one thing -- its mixer's
+            cache and the tail of a convolution in front of it, say.  The manager handles every member as a stream
+            of its own and hands out one view whose attributes are the members' views.
+
 A mixer gets a :class:`View` of its stream: the tensors by name (``view.k``, ``view.state``, ...) and,
 for a paged stream, ``group`` (the key of its block table and slot map in the step's context),
 ``page_tokens`` and ``window``.
@@ -23,7 +27,7 @@ for a paged stream, ``group`` (the key of its block table and slot map in the st
 from __future__ import annotations
 
 import dataclasses
-from typing import Dict, Tuple
+from typing import Any, Dict, Optional, Tuple
 
 
 @dataclasses.dataclass(frozen=True)
@@ -60,3 +64,41 @@ class FixedState:
 
     def slot_tensors(self) -> Dict[str, Tuple[Tuple[int, ...], str]]:
         return {"state": (tuple(self.shape), self.dtype)}
+
+
+@dataclasses.dataclass(frozen=True)
+class PagedLatent:
+    """One row of ``rank + rot`` numbers per token, in pages, shared by all heads: a low-rank latent from which keys
+    and values are made, followed by a rotated key part.  Rows lie ``[page, token, rank + rot]``.  ``window`` as for
+    :class:`PagedKV`."""
+    rank: int
+    rot: int
+    window: int = 0
+    per_token = True
+
+    def page_tensors(self, page_tokens: int) -> Dict[str, Tuple[int, ...]]:
+        return {"latent": (page_tokens, self.rank + self.rot)}
+
+    def group_key(self):
+        return ("window", self.window)
+
+    def first_kept(self, length: int) -> int:
+        return max(0, length - self.window + 1) if self.window > 0 else 0
+
+
+@dataclasses.dataclass(frozen=True)
+class States:
+    """Several per-request tensors of fixed size under names of their own: ``tensors`` is a tuple of
+    (name, shape, dtype name or None for the cache's own dtype).  Zeroed at admission like :class:`FixedState`."""
+    tensors: Tuple[Tuple[str, Tuple[int, ...], Optional[str]], ...]
+    per_token = False
+
+    def slot_tensors(self) -> Dict[str, Any]:
+        return {name: (tuple(shape), dtype) if dtype is not None else tuple(shape) for name, shape, dtype in self.tensors}
+
+
+@dataclasses.dataclass(frozen=True)
+class Bundle:
+    """What a layer keeps when it keeps more than one thing: ``members`` is a tuple of (name, spec), every spec one of
+    the kinds above (or None).  The layer's view has an attribute for every name."""
+    members: Tuple[Tuple[str, Any], ...]

@@ -4,3 +4,4 @@ from .registry import (  # noqa: F401
     load_config,
 )
 from .llama import LlamaConfig  # noqa: F401
+from .mamenex import MamenexConfig  # noqa: F401

@@ -55,6 +55,8 @@ def architecture_for(raw: Dict[str, Any]) -> Architecture:
     names = raw.get("architectures") or []
     if isinstance(names, str):
         names = [names]
+    if isinstance(raw.get("architecture"), str):      # (some configurations name one architecture, under this key)
+        names = list(names) + [raw["architecture"]]
     for n in names:
         if n in _BY_NAME:
             return _BY_NAME[n]

@@ -219,3 +219,49 @@ extern "C" {
 int bc4g_probe_read(const void* p, long bytes, float* sink, int workgroups, void* stream);
 int bc4g_probe_mfma(const void* operands, int iters, float* sink, int workgroups, void* stream);
 }
+
+extern "C" {
+// x[r, :] += y[r, :] * rsqrt(mean(y[r]^2) + eps) * w: the norm after a sublayer, added to the float residual stream
+// (w float32, as it multiplies; y float32 or bfloat16).
+int bc4g_rmsnorm_add(float* x, const void* y, int y_dtype, const float* w, int n_rows, int hidden, float eps, void* stream);
+// out = act(in) elementwise with act(z) = softplus(p) z^2 + z / 2 for z > 0 and (1/2 + softplus(q)) (e^z - 1 - z) + z / 2
+// otherwise; pq = (p, q) float32 on the device.
+int bc4g_xielu(const void* in, void* out, int dtype, const float* pq, long total, void* stream);
+
+// A causal convolution over time on each channel, across steps: out[t, c] = (add_input ? in[t, c] : 0) + out_bias[c] +
+// sum_j w[c, j] * input(t - taps + 1 + j)[c], where a row's input is in[row] + in_bias (rounded to the storage type) and
+// the inputs before a step's first row come from the request's state [slots, taps - 1, channels] (zero when the request
+// was admitted: zeros before the sequence).  Afterwards the state holds the request's last taps - 1 inputs.  The
+// step's rows are grouped by request: row_seq [T], seq_start [S + 1], seq_slots [S].  w, biases: float32.
+int bc4g_causal_conv(const void* in, int dtype, const float* in_bias, const float* w, const float* out_bias, int add_input,
+                     void* out, void* state, const int32_t* row_seq, const int32_t* seq_start, const int32_t* seq_slots,
+                     int n_rows, int n_seqs, int channels, int taps, void* stream);
+// The gates of the real-gated linear recurrent unit: u [T, width] in `blocks` equal parts; ra_t, ri_t
+// [blocks][in][out] (the block matrices transposed); decay = exp(-8 sigmoid(Ra u + ra_b) softplus(lam)),
+// drive = sqrt(1 - decay^2) sigmoid(Ri u + ri_b) u, both float32 [T, width].
+int bc4g_rglru_gates(const void* u, int dtype, const void* ra_t, const void* ri_t, int w_dtype, const float* ra_b,
+                     const float* ri_b, const float* lam, float* decay, float* drive, int n_rows, int width, int blocks,
+                     void* stream);
+// S_t = decay_t S_(t-1) + drive_t along every request's rows, from state [slots, width] (float32) and back into it;
+// out[t] = S_t * gelu_tanh(y[t] + y_bias).
+int bc4g_rglru_scan(const float* decay, const float* drive, const void* y, int dtype, const float* y_bias, void* out,
+                    float* state, const int32_t* seq_start, const int32_t* seq_slots, int n_rows, int n_seqs, int width,
+                    void* stream);
+
+// Latent attention (attention_latent.hip).  q [T, heads, plain + rot] and dkv [T, rank + rot] as projected; the row's
+// cache slot (slot_map[t] = page * page_tokens + offset; cache [pages, page_tokens, rank + rot]; null: nothing is
+// written) receives [rmsnorm(dkv[:rank]) * g | rotate(dkv[rank:])], and q_lat [T, heads, rank + rot] (float32) the
+// rotated part of every head's query in its last rot numbers.  Elements 2i and 2i + 1 of the first `dims` numbers of
+// a rotated part turn by position * base^(-2i / dims).
+int bc4g_latent_prepare(const void* q, const void* dkv, int dtype, const float* g, float eps, const int32_t* positions,
+                        const int32_t* slot_map, void* cache, float* q_lat, int n_rows, int heads, int plain, int rot,
+                        int rank, int dims, float base, void* stream);
+// out[t, h, :n] = w[h] a[t, h, :k] for every head: a at a + t * a_row + h * a_head, out likewise, w [heads, n, k].
+int bc4g_heads_gemm(const void* a, int a_dtype, long a_row, long a_head, const void* w, int w_dtype, void* out, int out_dtype,
+                    long o_row, long o_head, int m, int n, int k, int heads, void* stream);
+// out[t, h, :rank] = sum_j p_j cache[j, :rank] with p = exp(scale * q_lat[t, h] . cache[j]) over the keys the row sees
+// (max(0, p - window + 1) .. p), divided by their sum plus exp(sink[h]) (sink null: no such term).  float32 in and out.
+int bc4g_attention_latent(const float* q_lat, float* out, const void* cache, int dtype, const float* sink,
+                          const int32_t* block_table, int table_stride, const int32_t* row_seq, const int32_t* positions,
+                          int n_rows, int heads, int rank, int rot, int page_tokens, int window, float scale, void* stream);
+}

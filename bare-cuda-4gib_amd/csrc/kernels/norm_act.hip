@@ -1,0 +1,72 @@
+// A norm that is added to the residual stream (the second norm of a layer whose sublayers are normed on both
+// sides), and the xIELU activation.  One instantiation per storage type; all arithmetic in float.
+#include <math.h>
+
+#include "api.h"
+#include "common.h"
+
+namespace bc4g {
+namespace {
+
+constexpr int kBlock = 256;
+
+__device__ inline float softplus_f(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
+
+// x[r, :] += y[r, :] * rsqrt(mean(y[r]^2) + eps) * w.  The row of y is read twice (the second time from the cache).
+template <typename TY>
+__global__ __launch_bounds__(kBlock) void rmsnorm_add_kernel(float* __restrict__ x, const TY* __restrict__ y,
+                                                             const float* __restrict__ w, int hidden, float eps) {
+  __shared__ float scratch[16];
+  const TY* yr = y + static_cast<size_t>(blockIdx.x) * hidden;
+  float* xr = x + static_cast<size_t>(blockIdx.x) * hidden;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += kBlock) {
+    const float v = to_float(yr[i]);
+    ss += v * v;
+  }
+  const float scale = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(hidden) + eps);
+  for (int i = threadIdx.x; i < hidden; i += kBlock) xr[i] += to_float(yr[i]) * scale * w[i];
+}
+
+// act(z) = softplus(p) z^2 + z / 2 for z > 0, (1/2 + softplus(q)) (e^z - 1 - z) + z / 2 otherwise.
+template <typename T>
+__global__ void xielu_kernel(const T* __restrict__ in, T* __restrict__ out, const float* __restrict__ pq, long total) {
+  const float ap = softplus_f(pq[0]), aq = 0.5f + softplus_f(pq[1]);
+  const long stride = static_cast<long>(blockDim.x) * gridDim.x;
+  for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < total; i += stride) {
+    const float z = to_float(in[i]);
+    const float r = z > 0.f ? ap * z * z + 0.5f * z : aq * (expm1f(z) - z) + 0.5f * z;
+    out[i] = from_float<T>(r);
+  }
+}
+
+int grid_for(long total) {
+  const long g = (total + kBlock - 1) / kBlock;
+  return static_cast<int>(g < 1 ? 1 : (g > 65535 ? 65535 : g));
+}
+
+}  // namespace
+}  // namespace bc4g
+
+using namespace bc4g;
+
+extern "C" int bc4g_rmsnorm_add(float* x, const void* y, int y_dtype, const float* w, int n_rows, int hidden, float eps,
+                                void* stream) {
+  BC4G_REQUIRE(n_rows >= 0 && hidden > 0 && x && y && w, "rmsnorm_add: bad arguments rows=%d H=%d", n_rows, hidden);
+  if (n_rows == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (y_dtype == kF32) rmsnorm_add_kernel<float><<<n_rows, kBlock, 0, s>>>(x, static_cast<const float*>(y), w, hidden, eps);
+  else if (y_dtype == kBF16) rmsnorm_add_kernel<bf16_t><<<n_rows, kBlock, 0, s>>>(x, static_cast<const bf16_t*>(y), w, hidden, eps);
+  else return fail("rmsnorm_add: unknown dtype %d", y_dtype);
+  return check_launch("rmsnorm_add");
+}
+
+extern "C" int bc4g_xielu(const void* in, void* out, int dtype, const float* pq, long total, void* stream) {
+  BC4G_REQUIRE(total >= 0 && in && out && pq, "xielu: bad arguments (%ld elements)", total);
+  if (total == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == kF32) xielu_kernel<float><<<grid_for(total), kBlock, 0, s>>>(static_cast<const float*>(in), static_cast<float*>(out), pq, total);
+  else if (dtype == kBF16) xielu_kernel<bf16_t><<<grid_for(total), kBlock, 0, s>>>(static_cast<const bf16_t*>(in), static_cast<bf16_t*>(out), pq, total);
+  else return fail("xielu: unknown dtype %d", dtype);
+  return check_launch("xielu");
+}

@@ -1137,3 +1137,180 @@ def attention_work(ctx, n_heads: int, n_kv_heads: int, head_dim: int, window: in
     rows = 2 * ctx.n_tokens * n_heads * head_dim
     return (4.0 * pairs * n_heads * head_dim, (2 * keys * n_kv_heads * head_dim + rows) * elem,
             (2 * walked * n_kv_heads * head_dim + rows) * elem)
+
+
+# ---- a norm added to the stream, xIELU, state-carrying mixers, latent attention ----------------------------------------
+
+def _f32(what: str, name: str, t: Optional[torch.Tensor], shape) -> None:
+    if t is not None and (t.dtype != torch.float32 or tuple(t.shape) != tuple(shape)):
+        raise KernelError(f"{what}: {name} must be float32 {tuple(shape)}, got {t.dtype} {tuple(t.shape)}")
+
+
+def rmsnorm_add(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """x += y * rsqrt(mean(y^2) + eps) * weight, row by row, in place on the float residual stream x [T, H];
+    y [T, H] float32 or bfloat16, weight float32 [H] (as it multiplies)."""
+    _dev("rmsnorm_add", x, y, weight)
+    if x.dtype != torch.float32 or x.dim() != 2 or tuple(y.shape) != tuple(x.shape):
+        raise KernelError(f"rmsnorm_add: x must be float32 [T, H] and y of its shape, got {x.dtype} {tuple(x.shape)} and {tuple(y.shape)}")
+    n, hidden = x.shape
+    _f32("rmsnorm_add", "weight", weight, (hidden,))
+    library.call("bc4g_rmsnorm_add", _ptr(x), _ptr(y), _code(y, "rmsnorm_add"), _ptr(weight), n, hidden, float(eps), _stream(),
+                 cost=lambda: (5.0 * n * hidden, n * hidden * (8 + y.element_size())))
+    return x
+
+
+def xielu(z: torch.Tensor, pq: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """softplus(p) z^2 + z/2 for z > 0, (1/2 + softplus(q)) (e^z - 1 - z) + z/2 otherwise; pq = (p, q) float32 on the
+    device.  ``out`` may be z itself."""
+    _dev("xielu", z, pq, out)
+    _f32("xielu", "pq", pq, (2,))
+    if out is None:
+        out = torch.empty_like(z)
+    elif out.dtype != z.dtype or out.shape != z.shape:
+        raise KernelError("xielu: out must have the input's dtype and shape")
+    total = z.numel()
+    library.call("bc4g_xielu", _ptr(z), _ptr(out), _code(z, "xielu"), _ptr(pq), total, _stream(),
+                 cost=lambda: (6.0 * total, 2 * total * z.element_size()))
+    return out
+
+
+def _check_grouping(what: str, ctx, n_rows: int) -> None:
+    if ctx.n_tokens != n_rows:
+        raise KernelError(f"{what}: {n_rows} rows for a step of {ctx.n_tokens}")
+    _i32(what, "row_seq", ctx.row_seq, n_rows)
+    _i32(what, "seq_start", ctx.seq_start_dev, ctx.n_seqs + 1)
+    _i32(what, "seq_slots", ctx.seq_slots_dev, ctx.n_seqs)
+
+
+def causal_conv(x: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Tensor], ctx, in_bias: Optional[torch.Tensor] = None,
+                out_bias: Optional[torch.Tensor] = None, add_input: bool = False) -> torch.Tensor:
+    """A causal convolution over time on each channel of x [T, C], continued from every request's state
+    [slots, taps - 1, C] (x's dtype), which then receives the request's last taps - 1 inputs.  weight float32 [C, taps]
+    (its last column is the current token's); a row's input is x + in_bias; out_bias is added to the sum, and with
+    ``add_input`` x itself.  ``ctx``: the step's context (which rows belong to which request and slot)."""
+    _dev("causal_conv", x, weight, state, in_bias, out_bias)
+    if x.dim() != 2 or weight.dim() != 2 or weight.shape[0] != x.shape[1]:
+        raise KernelError(f"causal_conv: x {tuple(x.shape)} and weight {tuple(weight.shape)} do not match")
+    t, c = x.shape
+    taps = weight.shape[1]
+    _f32("causal_conv", "weight", weight, (c, taps))
+    _f32("causal_conv", "in_bias", in_bias, (c,))
+    _f32("causal_conv", "out_bias", out_bias, (c,))
+    if taps > 1:
+        if state is None or state.dtype != x.dtype or state.dim() != 3 or tuple(state.shape[1:]) != (taps - 1, c):
+            raise KernelError(f"causal_conv: state must be {x.dtype} [slots, {taps - 1}, {c}]")
+        if max(ctx.seq_slots, default=0) >= state.shape[0]:
+            raise KernelError(f"causal_conv: a slot beyond the state's {state.shape[0]}")
+    _check_grouping("causal_conv", ctx, t)
+    out = torch.empty_like(x)
+    library.call("bc4g_causal_conv", _ptr(x), _code(x, "causal_conv"), _ptr(in_bias), _ptr(weight), _ptr(out_bias),
+                 1 if add_input else 0, _ptr(out), _ptr(state), _ptr(ctx.row_seq), _ptr(ctx.seq_start_dev),
+                 _ptr(ctx.seq_slots_dev), t, ctx.n_seqs, c, taps, _stream(),
+                 cost=lambda: (2.0 * t * c * taps, 2 * t * c * x.element_size()))
+    return out
+
+
+def rglru(u: torch.Tensor, y: torch.Tensor, ra_t: torch.Tensor, ri_t: torch.Tensor, ra_b: torch.Tensor, ri_b: torch.Tensor,
+          lam: torch.Tensor, y_bias: Optional[torch.Tensor], state: torch.Tensor, ctx) -> torch.Tensor:
+    """The real-gated linear recurrent unit over a step's rows: u, y [T, W]; ra_t, ri_t [blocks, in, out] (the gates'
+    block matrices, transposed); biases and lam float32 [W]; state float32 [slots, W].  Gates, decay and state in
+    float32.  Returns S_t * gelu_tanh(y + y_bias) in u's dtype."""
+    _dev("rglru", u, y, ra_t, ri_t, ra_b, ri_b, lam, y_bias, state)
+    if u.dim() != 2 or y.shape != u.shape or y.dtype != u.dtype:
+        raise KernelError(f"rglru: u and y must be alike [T, W], got {tuple(u.shape)} and {tuple(y.shape)}")
+    t, w = u.shape
+    if ra_t.dim() != 3 or ra_t.shape != ri_t.shape or ra_t.dtype != ri_t.dtype or ra_t.shape[1] != ra_t.shape[2] \
+            or ra_t.shape[0] * ra_t.shape[1] != w:
+        raise KernelError(f"rglru: gate matrices {tuple(ra_t.shape)}, {tuple(ri_t.shape)} do not cut {w} channels into square blocks")
+    for name, v in (("ra_b", ra_b), ("ri_b", ri_b), ("lam", lam), ("y_bias", y_bias)):
+        _f32("rglru", name, v, (w,))
+    if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] != w or max(ctx.seq_slots, default=0) >= state.shape[0]:
+        raise KernelError(f"rglru: state must be float32 [slots, {w}] with a row for every slot of the step")
+    _check_grouping("rglru", ctx, t)
+    blocks, bs = ra_t.shape[0], ra_t.shape[1]
+    decay = torch.empty((t, w), dtype=torch.float32, device=u.device)
+    drive = torch.empty((t, w), dtype=torch.float32, device=u.device)
+    library.call("bc4g_rglru_gates", _ptr(u), _code(u, "rglru"), _ptr(ra_t), _ptr(ri_t), _code(ra_t, "rglru"), _ptr(ra_b),
+                 _ptr(ri_b), _ptr(lam), _ptr(decay), _ptr(drive), t, w, blocks, _stream(),
+                 cost=lambda: (4.0 * t * w * bs, 2 * w * bs * ra_t.element_size() + t * w * (u.element_size() + 8)))
+    out = torch.empty_like(u)
+    library.call("bc4g_rglru_scan", _ptr(decay), _ptr(drive), _ptr(y), _code(y, "rglru"), _ptr(y_bias), _ptr(out), _ptr(state),
+                 _ptr(ctx.seq_start_dev), _ptr(ctx.seq_slots_dev), t, ctx.n_seqs, w, _stream(),
+                 cost=lambda: (12.0 * t * w, t * w * (8 + 2 * u.element_size())))
+    return out
+
+
+LATENT_MAX_ROW = 640        # numbers of a latent cache row (latent + rotated key part) the attention kernel takes
+
+
+def latent_prepare(q: torch.Tensor, dkv: torch.Tensor, g: torch.Tensor, eps: float, positions: torch.Tensor,
+                   slot_map: Optional[torch.Tensor], cache: Optional[torch.Tensor], q_lat: torch.Tensor, heads: int, plain: int,
+                   rot: int, rank: int, dims: int, base: float) -> None:
+    """Writes [rmsnorm(dkv[:, :rank]) * g | rotate(dkv[:, rank:])] into every row's cache slot (``cache`` None: nowhere)
+    and every head's rotated query part into q_lat[:, h, rank:]."""
+    _dev("latent_prepare", q, dkv, g, positions, slot_map, cache, q_lat)
+    t = q.shape[0]
+    if q.dtype != dkv.dtype or tuple(q.shape) != (t, heads * (plain + rot)) or tuple(dkv.shape) != (t, rank + rot):
+        raise KernelError(f"latent_prepare: q {tuple(q.shape)} / dkv {tuple(dkv.shape)} do not fit heads={heads} plain={plain} rot={rot} rank={rank}")
+    _f32("latent_prepare", "g", g, (rank,))
+    _f32("latent_prepare", "q_lat", q_lat, (t, heads, rank + rot))
+    _i32("latent_prepare", "positions", positions, t)
+    if cache is not None:
+        if cache.dtype != q.dtype or cache.dim() != 3 or cache.shape[2] != rank + rot:
+            raise KernelError(f"latent_prepare: the cache must be {q.dtype} [pages, page_tokens, {rank + rot}], got {cache.dtype} {tuple(cache.shape)}")
+        _i32("latent_prepare", "slot_map", slot_map, t)
+    library.call("bc4g_latent_prepare", _ptr(q), _ptr(dkv), _code(q, "latent_prepare"), _ptr(g), float(eps), _ptr(positions),
+                 _ptr(slot_map) if cache is not None else None, _ptr(cache), _ptr(q_lat), t, heads, plain, rot, rank, int(dims),
+                 float(base), _stream(), cost=lambda: (4.0 * t * (rank + (heads + 1) * rot), t * (q.element_size() * (heads + 2) * rot + 2 * rank * q.element_size())))
+
+
+def heads_gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, k: int, n: int) -> None:
+    """out[t, h, :n] = w[h] a[t, h, :k] for a [T, heads, >= k], w [heads, n, k], out [T, heads, >= n] (the last
+    dimensions may be longer than k and n: parts of wider rows)."""
+    _dev("heads_gemm", a, w, out)
+    if a.dim() != 3 or out.dim() != 3 or w.dim() != 3 or a.shape[:2] != out.shape[:2] or a.shape[2] < k or out.shape[2] < n \
+            or tuple(w.shape) != (a.shape[1], n, k):
+        raise KernelError(f"heads_gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit k={k}, n={n}")
+    t, heads = a.shape[0], a.shape[1]
+    library.call("bc4g_heads_gemm", _ptr(a), _code(a, "heads_gemm"), heads * a.shape[2], a.shape[2], _ptr(w), _code(w, "heads_gemm"),
+                 _ptr(out), _code(out, "heads_gemm"), heads * out.shape[2], out.shape[2], t, n, k, heads, _stream(),
+                 cost=lambda: (2.0 * t * heads * n * k, heads * n * k * w.element_size() + t * heads * (k * a.element_size() + n * out.element_size())))
+
+
+def attention_latent(q_lat: torch.Tensor, cache: torch.Tensor, sink: Optional[torch.Tensor], block_table: torch.Tensor, ctx,
+                     heads: int, rank: int, rot: int, page_tokens: int, window: int, scale: float) -> torch.Tensor:
+    """Causal attention of every row over its request's latent cache rows; float32 [T, heads, rank] (the weighted
+    sums of the latents, before the values' up-projection)."""
+    _dev("attention_latent", q_lat, cache, sink, block_table)
+    t = q_lat.shape[0]
+    _f32("attention_latent", "q_lat", q_lat, (t, heads, rank + rot))
+    _f32("attention_latent", "sink", sink, (heads,))
+    if rank + rot > LATENT_MAX_ROW:
+        raise KernelError(f"attention_latent: a cache row of {rank + rot} numbers is beyond {LATENT_MAX_ROW}")
+    if cache.dim() != 3 or tuple(cache.shape[1:]) != (page_tokens, rank + rot):
+        raise KernelError(f"attention_latent: the cache must be [pages, {page_tokens}, {rank + rot}], got {tuple(cache.shape)}")
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or block_table.shape[0] < ctx.n_seqs:
+        raise KernelError("attention_latent: the block table must be int32 [requests, pages]")
+    if block_table.shape[1] * page_tokens < ctx.max_kv_len and not ctx.captured:
+        raise KernelError(f"attention_latent: the block table's {block_table.shape[1]} pages do not hold {ctx.max_kv_len} tokens")
+    _i32("attention_latent", "row_seq", ctx.row_seq, t)
+    _i32("attention_latent", "positions", ctx.positions, t)
+    out = torch.empty((t, heads, rank), dtype=torch.float32, device=q_lat.device)
+    library.call("bc4g_attention_latent", _ptr(q_lat), _ptr(out), _ptr(cache), _code(cache, "attention_latent"), _ptr(sink),
+                 _ptr(block_table), block_table.shape[1], _ptr(ctx.row_seq), _ptr(ctx.positions), t, heads, rank, rot, page_tokens,
+                 int(window), float(scale), _stream(), cost=lambda: attention_latent_work(ctx, heads, rank, rot, window, cache.element_size()))
+    return out
+
+
+def attention_latent_work(ctx, heads: int, rank: int, rot: int, window: int, elem: int):
+    """(operations, bytes to read at least) of latent attention over a step's rows."""
+    pairs = keys = 0
+    for s in range(ctx.n_seqs):
+        cached, new = int(ctx.seq_ctx[s]), int(ctx.seq_start[s + 1] - ctx.seq_start[s])
+        if window > 0:
+            pairs += sum(min(window, cached + i + 1) for i in range(new))
+            keys += min(cached + new, window + new - 1)
+        else:
+            pairs += new * cached + new * (new + 1) // 2
+            keys += cached + new
+    return 2.0 * pairs * heads * (2 * rank + rot), float(keys * (rank + rot) * elem)

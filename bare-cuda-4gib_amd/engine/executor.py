@@ -317,7 +317,12 @@ class Executor:
         for part in self._capture_parts:
             part.prepare_capture(S, bucket)
         ctx = self._context_from(dev, layout, group_layout, host)
-        self.model.forward(ctx)                      # once outside the graph: first-use work happens here
+        # Once outside the graph: first-use work happens here.  Keys and values written twice are the same keys and
+        # values; state that a step moves (a recurrence, a convolution's tail) must not move twice, so the requests'
+        # slots are put back as they were.
+        saved = self.cache.save_slots(host["seq_slots"])
+        self.model.forward(ctx)
+        self.cache.restore_slots(saved)
         torch.cuda.synchronize()
         ctx.made.clear()                             # what layers share is made again inside the graph
         graph = torch.cuda.CUDAGraph()

@@ -41,14 +41,16 @@ class Model:
         self.layers: List[Part] = []
         self._layer_bound: List[List[_Bound]] = []
         for ls in spec.layers:
-            mixer = _Bound(build_part("mixer", ls.mixer), ls.mixer)
-            ffn = _Bound(build_part("feedforward", ls.ffn), ls.ffn)
-            n1 = _Bound(build_part("norm", ls.mixer_norm), ls.mixer_norm)
-            n2 = _Bound(build_part("norm", ls.ffn_norm), ls.ffn_norm)
-            block = build_part("block", PartSpec(ls.block, dict(
-                mixer=mixer.part, ffn=ffn.part, mixer_norm=n1.part, ffn_norm=n2.part)))
-            self.layers.append(block)
-            self._layer_bound.append([n1, mixer, n2, ffn])
+            # the four parts every arrangement knows (a layer may lack the feed-forward and its norm), then
+            # whatever else this arrangement names
+            named = [("mixer_norm", "norm", ls.mixer_norm), ("mixer", "mixer", ls.mixer),
+                     ("ffn_norm", "norm", ls.ffn_norm), ("ffn", "feedforward", ls.ffn)]
+            named += [(name, category, ps) for name, (category, ps) in ls.extras.items()]
+            bound = {name: _Bound(build_part(category, ps), ps) for name, category, ps in named if ps is not None}
+            params = {name: None for name, _, ps in named[:4] if ps is None}
+            params.update({name: b.part for name, b in bound.items()})
+            self.layers.append(build_part("block", PartSpec(ls.block, params)))
+            self._layer_bound.append(list(bound.values()))
         self.schedule = list(spec.schedule)
         for e in self.schedule:
             if not (0 <= e.layer < len(self.layers)):
@@ -113,6 +115,12 @@ class Model:
         self.device_weight_bytes = torch.cuda.memory_allocated(rt.device) - before if cuda else self.weight_bytes
 
     # ---- cache --------------------------------------------------------------
+    def _cache_spec(self, layer: int):
+        """What the layer keeps: what its arrangement says (a block that keeps more than its mixer's cache), or its
+        mixer's."""
+        block = self.layers[layer]
+        return block.cache_spec() if hasattr(block, "cache_spec") else block.mixer.cache_spec()
+
     def cache_streams(self) -> Dict[Hashable, object]:
         """Cache stream id -> spec, from the schedule: the entry that writes a
         stream decides its spec; an entry may only read a stream that some
@@ -121,7 +129,7 @@ class Model:
         for e in self.schedule:
             if e.cache is None or not e.writes:
                 continue
-            spec = self.layers[e.layer].mixer.cache_spec()
+            spec = self._cache_spec(e.layer)
             if e.cache in streams and streams[e.cache] != spec:
                 raise ConfigError(f"cache stream {e.cache!r} is written with two different specs")
             streams[e.cache] = spec
@@ -133,7 +141,7 @@ class Model:
                 raise ConfigError(f"schedule entry for layer {e.layer} reads cache stream {e.cache!r}, "
                                   "which no entry writes")
             mixer = self.layers[e.layer].mixer
-            if mixer.cache_spec() != streams[e.cache]:
+            if self._cache_spec(e.layer) != streams[e.cache]:
                 raise ConfigError(f"layer {e.layer} uses cache stream {e.cache!r} with another spec than its writer")
             layout = mixer.cache_layout() if hasattr(mixer, "cache_layout") else None
             if layouts.setdefault(e.cache, layout) != layout:

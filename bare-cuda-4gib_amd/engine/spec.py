@@ -6,7 +6,7 @@ below it knows which architecture it came from.
 from __future__ import annotations
 
 import dataclasses
-from typing import Any, Dict, List, Optional
+from typing import Any, Dict, List, Optional, Tuple
 
 
 @dataclasses.dataclass
@@ -23,12 +23,16 @@ class PartSpec:
 @dataclasses.dataclass
 class LayerSpec:
     """One layer: an arrangement (``block``) of a mixer, a feed-forward and
-    their norms.  Every layer has its own, so layers of one model may differ."""
+    their norms.  Every layer has its own, so layers of one model may differ.
+    A layer may have no feed-forward (``ffn`` and ``ffn_norm`` None), and an
+    arrangement that has more parts than these four names them in ``extras``:
+    the block's own parameter name -> (category, PartSpec)."""
     block: str
     mixer: PartSpec
-    ffn: PartSpec
-    mixer_norm: PartSpec
-    ffn_norm: PartSpec
+    ffn: Optional[PartSpec] = None
+    mixer_norm: Optional[PartSpec] = None
+    ffn_norm: Optional[PartSpec] = None
+    extras: Dict[str, Tuple[str, PartSpec]] = dataclasses.field(default_factory=dict)
 
 
 @dataclasses.dataclass

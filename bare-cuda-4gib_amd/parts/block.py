@@ -1,6 +1,9 @@
 """How a layer's parts are arranged around the residual stream."""
 from __future__ import annotations
 
+import torch
+
+from ..cache.specs import Bundle
 from ..csrc import ops
 from .base import Part, register_part
 from .lazy import Normed
@@ -52,4 +55,42 @@ class PreNormBlock(Part):
         return norm.forward(x, ctx)
 
 
+class SandwichBlock(Part):
+    """Every sublayer normed on both sides: x += post(mixer(pre(x))); x += post(ffn(pre(x))).  The mixer may read
+    h + conv(h) instead of h = pre(x) (``mixer_conv``: a causal convolution over time whose tail is part of the
+    request's state), and a layer may have no feed-forward.  The sublayer's output is gathered in float32 and its
+    norm is added to the float32 stream in one kernel."""
+    category = "block"
+    graph_safe = True     # launches kernels only: may run inside a captured graph
+
+    def __init__(self, mixer, mixer_norm, mixer_post_norm, ffn=None, ffn_norm=None, ffn_post_norm=None, mixer_conv=None):
+        self.mixer, self.mixer_norm, self.mixer_post_norm = mixer, mixer_norm, mixer_post_norm
+        self.ffn, self.ffn_norm, self.ffn_post_norm, self.mixer_conv = ffn, ffn_norm, ffn_post_norm, mixer_conv
+
+    def children(self):
+        parts = [self.mixer_norm, self.mixer_conv, self.mixer, self.mixer_post_norm, self.ffn_norm, self.ffn, self.ffn_post_norm]
+        return [p for p in parts if p is not None]
+
+    def cache_spec(self):
+        """The mixer's cache, and beside it the tail of the convolution in front of the mixer."""
+        if self.mixer_conv is None:
+            return self.mixer.cache_spec()
+        return Bundle((("mixer", self.mixer.cache_spec()), ("conv", self.mixer_conv.cache_spec())))
+
+    def forward(self, x, ctx, cache, writes: bool = True) -> None:
+        h = self.mixer_norm.forward(x, ctx)
+        mixer_cache = cache
+        if self.mixer_conv is not None:
+            h = self.mixer_conv.forward(h, ctx, cache.conv, add_input=True)
+            mixer_cache = cache.mixer
+        y = torch.zeros_like(x)
+        self.mixer.forward(h, ctx, mixer_cache, y, writes)
+        self.mixer_post_norm.add_to(x, y)
+        if self.ffn is not None:
+            y = torch.zeros_like(x)
+            self.ffn.forward(self.ffn_norm.forward(x, ctx), ctx, y)
+            self.ffn_post_norm.add_to(x, y)
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "sandwich", SandwichBlock)

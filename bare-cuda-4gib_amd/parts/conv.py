@@ -1,0 +1,47 @@
+"""A short causal convolution over time on each channel, continued across a request's steps."""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..cache.specs import States
+from ..csrc import ops
+from ..errors import ConfigError
+from ..weights.loader import WeightSpec
+from .base import Part, register_part
+
+
+class CausalConv(Part):
+    """out[t, c] = bias[c] + sum_j w[c, j] * v[t - taps + 1 + j, c] over a request's rows v, zeros before its first
+    token; the last column of w is the current token's.  The request's last taps - 1 rows are its state (``tail``, in
+    the activations' dtype), so a prompt may be cut anywhere.  ``forward(v, ctx, view, add_input)`` returns the
+    convolution, with ``add_input`` v + the convolution."""
+    category = "conv"
+    graph_safe = True     # launches kernels only: may run inside a captured graph
+
+    def __init__(self, channels: int, taps: int, bias: bool = False):
+        if channels <= 0 or taps < 1:
+            raise ConfigError(f"causal convolution: {channels} channels and {taps} taps")
+        self.channels, self.taps, self.bias = int(channels), int(taps), bool(bias)
+        self.w = self.b = None
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        out = {"weight": WeightSpec((self.channels, self.taps), kind="vector")}
+        if self.bias:
+            out["bias"] = WeightSpec((self.channels,), kind="vector")
+        return out
+
+    def bind(self, tensors, rt) -> None:
+        self.w = tensors["weight"].to(torch.float32).contiguous()
+        self.b = tensors["bias"].to(torch.float32).contiguous() if self.bias else None
+
+    def cache_spec(self):
+        return States((("tail", (self.taps - 1, self.channels), None),))
+
+    def forward(self, v: torch.Tensor, ctx, view, add_input: bool = False, in_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return ops.causal_conv(v, self.w, view.tail if self.taps > 1 else None, ctx, in_bias=in_bias, out_bias=self.b,
+                               add_input=add_input)
+
+
+register_part("conv", "causal", CausalConv)

@@ -54,4 +54,30 @@ class SwiGLU(Part):
         linear(act, self.w_down, accumulate_into=residual, ctx=ctx)
 
 
+class DenseXIELU(Part):
+    """x += Wd act(Wu h), no biases, with act(z) = softplus(p) z^2 + z/2 for z > 0 and
+    (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2 otherwise; p and q are the two numbers of the tensor ``act``."""
+    category = "feedforward"
+    graph_safe = True     # launches kernels only: may run inside a captured graph
+
+    def __init__(self, hidden_size: int, intermediate_size: int):
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.w_up = self.w_down = self.pq = None
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        h, i = self.hidden_size, self.intermediate_size
+        return {"up": WeightSpec((i, h)), "down": WeightSpec((h, i)), "act": WeightSpec((2,), kind="vector")}
+
+    def bind(self, tensors, rt) -> None:
+        self.w_up = ops.StreamedWeight(tensors["up"])
+        self.w_down = ops.StreamedWeight(tensors["down"])
+        self.pq = tensors["act"].to(torch.float32).contiguous()
+        self.act_dtype = rt.act_dtype
+
+    def forward(self, h, ctx, residual) -> None:
+        z = linear(h, self.w_up, out_dtype=self.act_dtype)
+        linear(ops.xielu(z, self.pq, out=z), self.w_down, accumulate_into=residual, ctx=ctx)
+
+
 register_part("feedforward", "swiglu", SwiGLU)
+register_part("feedforward", "dense_xielu", DenseXIELU)

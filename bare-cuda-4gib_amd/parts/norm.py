@@ -1,5 +1,6 @@
 """RMSNorm: y = x * rsqrt(mean(x^2) + eps) * w, with eps on the mean square and
-sum and rsqrt in float (reference: engine/kernels/rmsnorm.cu:16-41)."""
+sum and rsqrt in float (reference: engine/kernels/rmsnorm.cu:16-41).  With ``offset`` the stored weight is
+counted from it: y = x * rsqrt(...) * (offset + w) -- a weight stored around zero has offset 1."""
 from __future__ import annotations
 
 from typing import Dict
@@ -15,16 +16,25 @@ class RMSNorm(Part):
     category = "norm"
     graph_safe = True
 
-    def __init__(self, size: int, eps: float):
-        self.size, self.eps = int(size), float(eps)
-        self.weight = None
+    def __init__(self, size: int, eps: float, offset: float = 0.0):
+        self.size, self.eps, self.offset = int(size), float(eps), float(offset)
+        self.weight = self._multiplier = None
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        return {"weight": WeightSpec((self.size,), kind="vector", init="ones")}
+        return {"weight": WeightSpec((self.size,), kind="vector", init="ones" if self.offset == 0.0 else "normal")}
 
     def bind(self, tensors, rt) -> None:
         self.weight = tensors["weight"]
+        if self.offset != 0.0:          # the sum in float32, whatever the weight is stored in
+            self.weight = (self.weight.to(torch.float32) + self.offset).contiguous()
+        self._multiplier = None
         self.out_dtype = rt.act_dtype
+
+    def add_to(self, x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+        """x += norm(y), in place on the float32 residual stream: the norm after a sublayer."""
+        if self._multiplier is None:
+            self._multiplier = self.weight.to(torch.float32).contiguous()
+        return ops.rmsnorm_add(x, y, self._multiplier, self.eps)
 
     def fusable(self):
         """What a product needs to absorb this norm: (scale vector, eps)."""
