@@ -47,6 +47,32 @@ SHAPES = {
                        num_key_value_heads=8, head_dim=128, intermediate_size=14336, rope_theta=500000.0,
                        max_position_embeddings=8192),
 }
+
+
+def mamenex_shape(width, layers, heads, dim, rot_dim, vdim, kv_rank, rwidth, blocks, ff, vocab=32000):
+    """A Mamenex configuration of real layer sizes: every third layer a recurrent one without a feed-forward, the
+    others latent attention with a dense feed-forward."""
+    att = dict(type="latent_attention", mlp=dict(kind="dense", ff=ff),
+               mixer=dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=kv_rank, scale=(dim + rot_dim) ** -0.5,
+                          rot=dict(base=10000.0, dims=rot_dim)))
+    rec = dict(type="rglru", mlp=None, mixer=dict(width=rwidth, blocks=blocks, conv=4))
+    return dict(architecture="Mamenex", vocab=vocab, width=width, norm=dict(eps=1e-5), canon=dict(taps=3),
+                layers=[rec if i % 3 == 0 else att for i in range(layers)])
+
+
+# --only mamenex: the design at a few sizes that resemble a real model's layers, each beside the Llama decoder of the
+# same width, depth, head count and feed-forward parameters (SwiGLU's three matrices of 2/3 the width of the dense two).
+MAMENEX_SIZES = {
+    "1k": (mamenex_shape(1024, 6, 8, 64, 32, 64, 224, 1024, 8, 4096),
+           dict(TINYLLAMA, tie_word_embeddings=True, max_position_embeddings=8192, hidden_size=1024, num_hidden_layers=6, num_attention_heads=8, num_key_value_heads=2, head_dim=128,
+                intermediate_size=2752)),
+    "2k": (mamenex_shape(2048, 6, 16, 128, 64, 128, 512, 2560, 10, 8192),
+           dict(TINYLLAMA, tie_word_embeddings=True, max_position_embeddings=8192, hidden_size=2048, num_hidden_layers=6, num_attention_heads=16, num_key_value_heads=4, head_dim=128,
+                intermediate_size=5504)),
+    "4k": (mamenex_shape(4096, 6, 32, 128, 64, 128, 512, 4096, 16, 14336),
+           dict(TINYLLAMA, tie_word_embeddings=True, max_position_embeddings=8192, hidden_size=4096, num_hidden_layers=6, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+                intermediate_size=9600)),
+}
 BASELINE_DECODE_B1 = 77.3                   # the reference's only FP16 decode number (batch 1, RTX 3050)
 
 
@@ -55,7 +81,7 @@ def build_model(layers, dtype, seed=0, shape=TINYLLAMA):
     from bare_cuda_4gib_amd.config import architecture_for
     from bare_cuda_4gib_amd.engine import Model, Runtime, parse_dtype
     from bare_cuda_4gib_amd.weights.random_device import random_tensors_on_device
-    raw = dict(shape, num_hidden_layers=layers)
+    raw = dict(shape, num_hidden_layers=layers) if layers is not None else dict(shape)
     arch = architecture_for(raw)
     cfg = arch.config_class.from_dict(raw)
     model = Model(arch.describe(cfg))
@@ -162,6 +188,81 @@ def run_prefill(model, cfg, tokens, runs=3, seed=2):
     del ex
     torch.cuda.empty_cache()
     return best
+
+
+def kernel_table(model, cfg, prefill_tokens, batch, context, dtype):
+    """Per kernel of one prompt and of eight decode steps, launched one by one with the profiler on: calls, time, and
+    how far the kernel is from the roofline of the work its caller states (the larger of operations / the matrix
+    cores' peak and bytes / HBM's)."""
+    import torch
+    from bare_cuda_4gib_amd.csrc.profile import profiler
+    from bare_cuda_4gib_amd.engine import Executor, StepEntry
+    page, prof = 64, profiler()
+    pages_each = -(-(max(prefill_tokens, context) + 16) // page)
+    ex = Executor(model, num_pages=pages_each * batch, max_requests=batch, max_tokens=pages_each * page, page_tokens=page,
+                  use_graphs=False)
+    gen = torch.Generator().manual_seed(7)
+    ids = lambda n: torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist()      # noqa: E731
+    out = {}
+
+    def table():
+        rows = []
+        for st in prof.stats():
+            roof_ms = max(st.flops / (PEAK_TFLOPS[dtype] * 1e12), st.bytes / (HBM_PEAK_GBS * 1e9)) * 1e3
+            rows.append({"kernel": st.name, "calls": st.calls, "ms": round(st.ms, 4),
+                         "bound": "flops" if st.flops / (PEAK_TFLOPS[dtype] * 1e12) > st.bytes / (HBM_PEAK_GBS * 1e9) else "bytes",
+                         "of_roofline": round(roof_ms / st.ms, 4) if st.ms > 0 else None})
+        return rows
+    ex.admit("w")
+    ex.step([StepEntry("w", ids(prefill_tokens), [prefill_tokens - 1])])       # once unprofiled: first-use work
+    ex.release("w")
+    prof.reset()
+    prof.enable(True)
+    ex.admit("p")
+    ex.step([StepEntry("p", ids(prefill_tokens), [prefill_tokens - 1])])
+    out["prefill"] = table()
+    prof.enable(False)
+    ex.release("p")
+    for b in range(batch):
+        ex.admit(b)
+        ex.step([StepEntry(b, ids(context), [context - 1])])
+    step = [StepEntry(b, [1], [0]) for b in range(batch)]
+    ex.step(step)
+    prof.reset()
+    prof.enable(True)
+    for _ in range(8):
+        ex.step(step)
+    out["decode"] = table()
+    prof.enable(False)
+    prof.reset()
+    del ex
+    torch.cuda.empty_cache()
+    return out
+
+
+def run_mamenex(size, args):
+    """Prefill and decode of the design at one size beside the Llama decoder of equal size; with --kernels the
+    per-kernel tables of both."""
+    dtype = "bfloat16" if args.dtype == "bf16" else "float32"
+    elem = 2 if args.dtype == "bf16" else 4
+    line = {"only": "mamenex", "size": size, "dtype": args.dtype, "prefill_tokens": args.prefill_tokens, "batch": args.batch,
+            "prompt_len": args.prompt_len}
+    for name, shape in zip(("mamenex", "llama"), MAMENEX_SIZES[size]):
+        import torch
+        model, cfg = build_model(None, dtype, shape=shape)
+        pre_s = run_prefill(model, cfg, args.prefill_tokens)
+        dt, contexts = run_decode(model, cfg, args.batch, args.prompt_len, args.steps, args.warmup)
+        gbs = decode_bytes(model, elem, contexts) / (dt / args.steps) / 1e9
+        line[name] = {"weights_mb": round(model.weight_bytes / 2 ** 20, 1),
+                      "prefill_ms": round(pre_s * 1e3, 3), "prefill_tokens_per_s": round(args.prefill_tokens / pre_s, 1),
+                      "prefill_frac": round(prefill_flops(model, args.prefill_tokens) / pre_s / (PEAK_TFLOPS[args.dtype] * 1e12), 4),
+                      "decode_ms_per_step": round(dt / args.steps * 1e3, 4), "decode_tokens_per_s": round(args.batch * args.steps / dt, 1),
+                      "decode_hbm_frac": round(gbs / HBM_PEAK_GBS, 4)}
+        if args.kernels:
+            line[name]["kernels"] = kernel_table(model, cfg, args.prefill_tokens, args.batch, args.prompt_len, args.dtype)
+        del model
+        torch.cuda.empty_cache()
+    return line
 
 
 def run_gemm(m, n, k, runs=20):
@@ -309,7 +410,9 @@ def main() -> int:
     ap.add_argument("--top-p", type=float, default=1.0, help="--only serve: ... and this top-p (1: none)")
     ap.add_argument("--gather-ms", type=float, default=0.0,
                     help="--only chat: the scheduler waits this long before it admits those who came while others decode")
-    ap.add_argument("--only", choices=["decode", "prefill", "serve", "chat", "gemm", "peaks"], default=None,
+    ap.add_argument("--sizes", default="1k,2k,4k", help="--only mamenex: which of the sizes " + ", ".join(MAMENEX_SIZES))
+    ap.add_argument("--kernels", action="store_true", help="--only mamenex: add the per-kernel tables (time, part of the roofline)")
+    ap.add_argument("--only", choices=["decode", "prefill", "serve", "chat", "gemm", "peaks", "mamenex"], default=None,
                     help="run one part only and print its own short line (for profiling); peaks: what a kernel that only "
                          "reads, and one of nothing but matrix-core instructions, reach on this device")
     ap.add_argument("--mnk", default="2048,11264,2048",
@@ -325,6 +428,10 @@ def main() -> int:
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     if args.only == "gemm":
         print(json.dumps(run_gemm(*(int(v) for v in args.mnk.split(",")))), flush=True)
+        return 0
+    if args.only == "mamenex":
+        for size in args.sizes.split(","):
+            print(json.dumps(run_mamenex(size, args)), flush=True)
         return 0
     from bare_cuda_4gib_amd.csrc.peaks import measured_peaks
     measured = measured_peaks()
