@@ -264,4 +264,14 @@ int bc4g_heads_gemm(const void* a, int a_dtype, long a_row, long a_head, const v
 int bc4g_attention_latent(const float* q_lat, float* out, const void* cache, int dtype, const float* sink,
                           const int32_t* block_table, int table_stride, const int32_t* row_seq, const int32_t* positions,
                           int n_rows, int heads, int rank, int rot, int page_tokens, int window, float scale, void* stream);
+// The same on the matrix cores for a bfloat16 cache (attention_latent_mfma.hip): rank + rot a multiple of 32 up to 576,
+// rank a multiple of 16 up to 512 (bc4g_attention_latent_mfma_takes).  The step's rows are grouped by request (seq_start
+// [S + 1], seq_ctx [S]: tokens cached before the step); most_tokens: the most rows one request brings.  n_splits > 1 cuts
+// every walk over the keys into that many parts over workgroups, merged from part_o [n_splits, T, heads, rank] and
+// part_ml [n_splits, T, heads, 2] (float32).
+int bc4g_attention_latent_mfma_takes(int rank, int rot);
+int bc4g_attention_latent_mfma(const float* q_lat, float* out, float* part_o, float* part_ml, const void* cache,
+                               const float* sink, const int32_t* block_table, int table_stride, const int32_t* seq_start,
+                               const int32_t* seq_ctx, int n_seqs, int n_tokens, int most_tokens, int heads, int rank, int rot,
+                               int page_tokens, int window, float scale, int n_splits, void* stream);
 }

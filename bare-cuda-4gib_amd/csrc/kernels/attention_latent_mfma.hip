@@ -1,0 +1,248 @@
+// Latent attention on the matrix cores (bfloat16 cache; see attention_latent.hip for what is computed).
+//
+// All heads read the same cache rows, so the 16 columns of a matrix-core tile are (token, head) pairs of one request:
+// hb = min(heads, 16) heads of 16 / hb consecutive tokens.  A wave takes one such tile, a workgroup four tiles that
+// follow each other (the head groups of one token block first, then the next token block), and the four walk the
+// request's keys together: a tile of 32 cache rows goes into LDS once for all of them.
+//
+//   scores   S^T[keys x queries] = K[keys x row] Q^T[row x queries]: the cache rows are the A operand as they lie in
+//            LDS (16 bytes a lane), the queries the B operand, kept in registers for the whole walk; a lane then
+//            holds, for its query, eight of the 32 keys, so maximum and sum of a query are in-lane plus two lane swaps
+//   output   O^T[latent x queries] += V^T[latent x keys] P^T[keys x queries] with V = the first `rank` numbers of the
+//            same LDS rows: the weights go from the score registers straight into the B operand (which key a k-slot
+//            stands for is free, as long as A agrees), and the A operand gathers its eight keys of one latent number
+//            from LDS two bytes at a time
+//
+// The keys may be cut into n_splits parts over workgroups (few rows over a long context: a decode step), whose
+// unnormalised float partials a second kernel merges; the sink joins the sum where the sum is finished.
+#include <float.h>
+#include <math.h>
+
+#include "api.h"
+#include "common.h"
+#include "mfma.h"
+
+namespace bc4g {
+namespace {
+
+constexpr int kKeys = 32;                   // cache rows a key tile holds
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ inline unsigned pack_bf16(float lo, float hi) {
+  return static_cast<unsigned>(bf16_bits_from_float(lo)) | (static_cast<unsigned>(bf16_bits_from_float(hi)) << 16);
+}
+
+// KS: k-steps of 32 over a cache row (dk <= 32 KS); DB: blocks of 16 over the latent (rank <= 16 DB).
+template <int KS, int DB>
+__global__ __launch_bounds__(256) void latent_mfma_kernel(
+    const float* __restrict__ q_lat, float* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const bf16_t* __restrict__ cache, const float* __restrict__ sink, const int32_t* __restrict__ block_table,
+    int table_stride, const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_ctx, int n_tokens, int heads,
+    int rank, int dk, int page_tokens, int window, float scale, int hb, int tpt, int n_hg, int n_splits) {
+  extern __shared__ uint4 tile[];                             // [kKeys][dk / 8 + 1] pieces of 16 bytes
+  const int s = blockIdx.y, z = blockIdx.z;
+  const int tok0 = seq_start[s], n_tok = seq_start[s + 1] - tok0, cached = seq_ctx[s];
+  const int n_tb = (n_tok + tpt - 1) / tpt, n_tiles = n_tb * n_hg;
+  const int tile0 = blockIdx.x * 4;
+  if (tile0 >= n_tiles) return;                               // (the whole workgroup)
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int my_tile = tile0 + wave;
+  const bool wave_live = my_tile < n_tiles;
+  const int tb = wave_live ? my_tile / n_hg : 0, hg = wave_live ? my_tile % n_hg : 0;
+  const int c = lane % 16, g = lane / 16;
+  const int tq = tb * tpt + c / hb, head = hg * hb + c % hb;
+  const bool q_live = wave_live && c / hb < tpt && tq < n_tok && head < heads;
+  const int pos = cached + tq;
+  const int32_t* table = block_table + static_cast<long>(s) * table_stride;
+  const int cpr = dk / 8, pitch = cpr + 1;                    // 16-byte pieces of a row; of a row in LDS
+
+  // the keys this workgroup's rows see, in tiles aligned to multiples of 32, and this part's share of them
+  const int tb_last = min(n_tb - 1, (tile0 + 3) / n_hg);
+  const int last_pos = cached + min(n_tok, (tb_last + 1) * tpt) - 1;
+  const int first_pos = window > 0 ? max(0, cached + (tile0 / n_hg) * tpt - window + 1) : 0;
+  const int kt_begin = first_pos / kKeys, kt_end = last_pos / kKeys + 1;
+  const int per = (kt_end - kt_begin + n_splits - 1) / n_splits;
+  const int kt_lo = kt_begin + z * per, kt_hi = min(kt_end, kt_lo + per);
+
+  uint4 qf[KS];
+  {
+    const float* qrow = q_lat + (static_cast<long>(tok0 + tq) * heads + head) * dk;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      qf[ks] = zero16();
+      if (q_live && ks * 32 < dk) {
+        const float4 a = *reinterpret_cast<const float4*>(qrow + ks * 32 + 8 * g);
+        const float4 b = *reinterpret_cast<const float4*>(qrow + ks * 32 + 8 * g + 4);
+        qf[ks] = make_uint4(pack_bf16(a.x, a.y), pack_bf16(a.z, a.w), pack_bf16(b.x, b.y), pack_bf16(b.z, b.w));
+      }
+    }
+  }
+  floatx4 acc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) acc[db] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const float scale2 = scale * kLog2e;                        // exponents to the base 2
+  const uint16_t* tile16 = reinterpret_cast<const uint16_t*>(tile);
+  const int pitch16 = pitch * 8;
+
+  for (int kt = kt_lo; kt < kt_hi; ++kt) {
+    const int j0 = kt * kKeys;
+    __syncthreads();                                          // the tile before has been read by everyone
+    for (int piece = threadIdx.x; piece < kKeys * cpr; piece += 256) {
+      const int key = piece / cpr, part = piece - key * cpr;
+      const int j = j0 + key;
+      uint4 v = zero16();
+      if (j >= first_pos && j <= last_pos) {
+        const long page = table[j / page_tokens];
+        v = load16(cache + (page * page_tokens + j % page_tokens) * dk + part * 8);
+      }
+      tile[key * pitch + part] = v;
+    }
+    __syncthreads();
+    if (!wave_live) continue;
+    floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks * 32 < dk) {
+        s0 = mfma_16x16x32(tile[c * pitch + ks * 4 + g], qf[ks], s0);
+        s1 = mfma_16x16x32(tile[(16 + c) * pitch + ks * 4 + g], qf[ks], s1);
+      }
+    }
+    // this lane's eight keys of its query: j0 + 4g + i and j0 + 16 + 4g + i
+    float p[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int j = j0 + (i < 4 ? 0 : 16) + 4 * g + (i & 3);
+      const bool seen = q_live && j <= pos && (window == 0 || j > pos - window);
+      p[i] = seen ? (i < 4 ? s0[i] : s1[i - 4]) * scale2 : -INFINITY;
+      mx = fmaxf(mx, p[i]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    const float m_new = fmaxf(m, mx);
+    const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m - m_new);     // (m = -inf: 0)
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      p[i] = p[i] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(p[i] - m_new);
+      sum += p[i];
+    }
+    l = l * alpha + sum;
+    m = m_new;
+    if (__any(alpha != 1.f)) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db) acc[db] *= alpha;
+    }
+    const uint4 pf = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
+    const uint16_t* col = tile16 + (4 * g) * pitch16 + c;     // key 4g, latent number c of a block
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      if (db * 16 < rank) {
+        const uint16_t* v = col + db * 16;
+        const uint4 a = make_uint4(
+            v[0] | (static_cast<unsigned>(v[pitch16]) << 16), v[2 * pitch16] | (static_cast<unsigned>(v[3 * pitch16]) << 16),
+            v[16 * pitch16] | (static_cast<unsigned>(v[17 * pitch16]) << 16),
+            v[18 * pitch16] | (static_cast<unsigned>(v[19 * pitch16]) << 16));
+        acc[db] = mfma_16x16x32(a, pf, acc[db]);
+      }
+    }
+  }
+  if (!q_live) return;
+  l += __shfl_xor(l, 16, kWave);
+  l += __shfl_xor(l, 32, kWave);
+  const long row = static_cast<long>(tok0 + tq) * heads + head;
+  if (n_splits == 1) {
+    if (sink) l += __builtin_amdgcn_exp2f(sink[head] * kLog2e - m);
+    const float inv = 1.0f / l;
+    float* o = out + row * rank;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+      if (db * 16 < rank)
+        *reinterpret_cast<float4*>(o + db * 16 + 4 * g) = make_float4(acc[db][0] * inv, acc[db][1] * inv, acc[db][2] * inv, acc[db][3] * inv);
+  } else {
+    float* o = part_o + (static_cast<long>(z) * n_tokens * heads + row) * rank;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+      if (db * 16 < rank)
+        *reinterpret_cast<float4*>(o + db * 16 + 4 * g) = make_float4(acc[db][0], acc[db][1], acc[db][2], acc[db][3]);
+    if (g == 0) {
+      float* ml = part_ml + (static_cast<long>(z) * n_tokens * heads + row) * 2;
+      ml[0] = m;
+      ml[1] = l;
+    }
+  }
+}
+
+// out[row] = sum_z part_o[z][row] 2^(m_z - M) / (sum_z l_z 2^(m_z - M) + 2^(sink log2(e) - M)): one wave a (row, head).
+__global__ __launch_bounds__(kWave) void latent_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                             const float* __restrict__ sink, float* __restrict__ out,
+                                                             long rows, int heads, int rank, int n_splits) {
+  const long row = blockIdx.x;
+  float big = -INFINITY;
+  for (int z = 0; z < n_splits; ++z) big = fmaxf(big, part_ml[(z * rows + row) * 2]);
+  float total = sink ? __builtin_amdgcn_exp2f(sink[row % heads] * kLog2e - big) : 0.f;
+  for (int z = 0; z < n_splits; ++z) {
+    const float* ml = part_ml + (z * rows + row) * 2;
+    total += ml[1] * __builtin_amdgcn_exp2f(ml[0] - big);
+  }
+  const float inv = 1.0f / total;
+  for (int d = threadIdx.x; d < rank; d += kWave) {
+    float sum = 0.f;
+    for (int z = 0; z < n_splits; ++z)
+      sum += part_o[(z * rows + row) * rank + d] * __builtin_amdgcn_exp2f(part_ml[(z * rows + row) * 2] - big);
+    out[row * rank + d] = sum * inv;
+  }
+}
+
+}  // namespace
+}  // namespace bc4g
+
+using namespace bc4g;
+
+// Whether the matrix-core kernel takes these sizes (a bfloat16 cache): cache rows of whole k-steps, a latent of whole
+// blocks, both within what a wave's registers hold.
+extern "C" int bc4g_attention_latent_mfma_takes(int rank, int rot) {
+  const int dk = rank + rot;
+  return dk % 32 == 0 && rank % 16 == 0 && dk <= 576 && rank <= 512 && rank > 0;
+}
+
+// q_lat [T, heads, rank + rot] float32; out [T, heads, rank] float32; cache bfloat16 [pages, page_tokens, rank + rot].
+// n_tiles_most: the most (token block, head group) tiles a request of the step has; n_splits > 1 needs part_o
+// [n_splits, T, heads, rank] and part_ml [n_splits, T, heads, 2].
+extern "C" int bc4g_attention_latent_mfma(const float* q_lat, float* out, float* part_o, float* part_ml, const void* cache,
+                                          const float* sink, const int32_t* block_table, int table_stride,
+                                          const int32_t* seq_start, const int32_t* seq_ctx, int n_seqs, int n_tokens,
+                                          int most_tokens, int heads, int rank, int rot, int page_tokens, int window,
+                                          float scale, int n_splits, void* stream) {
+  BC4G_REQUIRE(n_seqs >= 0 && n_tokens >= 0 && heads > 0 && most_tokens >= 0 && bc4g_attention_latent_mfma_takes(rank, rot),
+               "attention_latent_mfma: sizes it does not take (S=%d T=%d heads=%d rank=%d rot=%d)", n_seqs, n_tokens, heads, rank, rot);
+  BC4G_REQUIRE(page_tokens > 0 && table_stride > 0 && window >= 0 && n_splits >= 1 && n_splits <= 64,
+               "attention_latent_mfma: bad cache sizes or parts (page_tokens=%d table_stride=%d window=%d parts=%d)", page_tokens,
+               table_stride, window, n_splits);
+  BC4G_REQUIRE(q_lat && out && cache && block_table && seq_start && seq_ctx && (n_splits == 1 || (part_o && part_ml)),
+               "attention_latent_mfma: a tensor is missing");
+  BC4G_REQUIRE(reinterpret_cast<uintptr_t>(cache) % 16 == 0 && reinterpret_cast<uintptr_t>(q_lat) % 16 == 0 &&
+               reinterpret_cast<uintptr_t>(out) % 16 == 0, "attention_latent_mfma: operands must lie on 16-byte boundaries");
+  if (n_tokens == 0 || n_seqs == 0 || most_tokens == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int dk = rank + rot;
+  const int hb = heads < 16 ? heads : 16, tpt = 16 / hb, n_hg = ceil_div(heads, hb);
+  const int most_tiles = ceil_div(most_tokens, tpt) * n_hg;
+  BC4G_REQUIRE(n_seqs <= 65535 && n_splits <= 65535, "attention_latent_mfma: %d requests are beyond the grid limit", n_seqs);
+  dim3 grid(ceil_div(most_tiles, 4), n_seqs, n_splits);
+  const size_t lds = static_cast<size_t>(kKeys) * (dk / 8 + 1) * 16;
+  const bf16_t* kc = static_cast<const bf16_t*>(cache);
+#define BC4G_LATENT(KS, DB)                                                                                                 \
+  latent_mfma_kernel<KS, DB><<<grid, 256, lds, s>>>(q_lat, out, part_o, part_ml, kc, sink, block_table, table_stride, seq_start, \
+                                                    seq_ctx, n_tokens, heads, rank, dk, page_tokens, window, scale, hb, tpt, n_hg, \
+                                                    n_splits)
+  if (dk <= 128 && rank <= 64) BC4G_LATENT(4, 4);
+  else if (dk <= 320 && rank <= 256) BC4G_LATENT(10, 16);
+  else BC4G_LATENT(18, 32);
+#undef BC4G_LATENT
+  if (n_splits > 1)
+    latent_merge_kernel<<<static_cast<unsigned>(static_cast<long>(n_tokens) * heads), kWave, 0, s>>>(
+        part_o, part_ml, sink, out, static_cast<long>(n_tokens) * heads, heads, rank, n_splits);
+  return check_launch("attention_latent_mfma");
+}

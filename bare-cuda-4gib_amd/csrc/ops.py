@@ -1241,6 +1241,30 @@ def rglru(u: torch.Tensor, y: torch.Tensor, ra_t: torch.Tensor, ri_t: torch.Tens
 
 
 LATENT_MAX_ROW = 640        # numbers of a latent cache row (latent + rotated key part) the attention kernel takes
+LATENT_MFMA = True          # (off: the plain kernel also where the matrix-core kernel takes the sizes)
+LATENT_ENOUGH_GROUPS = 256  # workgroups from which on the keys are not cut into parts
+LATENT_MAX_SPLITS = 64
+
+
+def attention_latent_mfma_takes(cache: torch.Tensor, rank: int, rot: int) -> bool:
+    """Whether the matrix-core kernel serves this cache: bfloat16, rows of whole k-steps of 32, a latent of whole
+    blocks of 16, within what a wave's registers hold."""
+    dk = rank + rot
+    return (LATENT_MFMA and cache.dtype == torch.bfloat16 and dk % 32 == 0 and rank % 16 == 0 and dk <= 576 and 0 < rank <= 512
+            and cache.data_ptr() % 16 == 0)
+
+
+def latent_splits(seq_start, heads: int, max_kv_len: int) -> int:
+    """Into how many parts the matrix-core kernel cuts every walk over the keys: one where the step's rows fill the
+    GPU by themselves (a workgroup takes four tiles of 16 (token, head) pairs of one request), else as many as bring
+    the workgroups to twice that, while a part keeps two key tiles of 32."""
+    hb = min(heads, 16)
+    tpt, n_hg = 16 // hb, -(-heads // hb)
+    groups = sum(-(-(-(-int(seq_start[s + 1] - seq_start[s]) // tpt) * n_hg) // 4) for s in range(len(seq_start) - 1))
+    if groups >= LATENT_ENOUGH_GROUPS or groups == 0:
+        return 1
+    key_tiles = -(-max_kv_len // 32)
+    return max(1, min(-(-2 * LATENT_ENOUGH_GROUPS // groups), key_tiles // 2, LATENT_MAX_SPLITS))
 
 
 def latent_prepare(q: torch.Tensor, dkv: torch.Tensor, g: torch.Tensor, eps: float, positions: torch.Tensor,
@@ -1296,6 +1320,20 @@ def attention_latent(q_lat: torch.Tensor, cache: torch.Tensor, sink: Optional[to
     _i32("attention_latent", "row_seq", ctx.row_seq, t)
     _i32("attention_latent", "positions", ctx.positions, t)
     out = torch.empty((t, heads, rank), dtype=torch.float32, device=q_lat.device)
+    if attention_latent_mfma_takes(cache, rank, rot):
+        _i32("attention_latent", "seq_start", ctx.seq_start_dev, ctx.n_seqs + 1)
+        _i32("attention_latent", "seq_ctx", ctx.seq_ctx_dev, ctx.n_seqs)
+        n_splits = latent_splits(ctx.seq_start, heads, ctx.max_kv_len)
+        most = max(int(ctx.seq_start[s + 1] - ctx.seq_start[s]) for s in range(ctx.n_seqs))
+        part_o = part_ml = None
+        if n_splits > 1:
+            part_o = torch.empty((n_splits, t, heads, rank), dtype=torch.float32, device=q_lat.device)
+            part_ml = torch.empty((n_splits, t, heads, 2), dtype=torch.float32, device=q_lat.device)
+        library.call("bc4g_attention_latent_mfma", _ptr(q_lat), _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(cache), _ptr(sink),
+                     _ptr(block_table), block_table.shape[1], _ptr(ctx.seq_start_dev), _ptr(ctx.seq_ctx_dev), ctx.n_seqs, t, most,
+                     heads, rank, rot, page_tokens, int(window), float(scale), n_splits, _stream(),
+                     cost=lambda: attention_latent_work(ctx, heads, rank, rot, window, cache.element_size()))
+        return out
     library.call("bc4g_attention_latent", _ptr(q_lat), _ptr(out), _ptr(cache), _code(cache, "attention_latent"), _ptr(sink),
                  _ptr(block_table), block_table.shape[1], _ptr(ctx.row_seq), _ptr(ctx.positions), t, heads, rank, rot, page_tokens,
                  int(window), float(scale), _stream(), cost=lambda: attention_latent_work(ctx, heads, rank, rot, window, cache.element_size()))

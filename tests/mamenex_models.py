@@ -29,7 +29,8 @@ def recurrent(width, blocks, conv, ff=None):
 # Configurations that differ in every size and constant: rotated dimensions fewer than the rotated part (P) or all
 # of it, one head (P) and several, one gate block (P, R) and several, convolutions of one tap (P: the recurrent
 # layer's; R: the one in front of the mixers), a latent row longer than a wave (Q: 72 + 24, R: 130 + 6, no multiple
-# of four), layers with and without a feed-forward after either mixer, an odd vocabulary.
+# of four), layers with and without a feed-forward after either mixer, an odd vocabulary; S has latent rows of whole
+# matrix-core steps (48 + 16, 112 + 16) with four heads and with twenty (more than a tile's sixteen columns).
 CONFIGS: Dict[str, dict] = {
     "P": dict(architecture="Mamenex", vocab=96, width=48, norm=dict(eps=1e-6), canon=dict(taps=2), layers=[
         recurrent(40, 5, 3, ff=80),
@@ -43,8 +44,12 @@ CONFIGS: Dict[str, dict] = {
     "R": dict(architecture="Mamenex", vocab=77, width=40, norm=dict(eps=1e-3), canon=dict(taps=1), layers=[
         recurrent(36, 1, 2, ff=44),
         latent(2, 10, 6, 12, 130, dims=2, base=50.0)]),
+    "S": dict(architecture="Mamenex", vocab=200, width=64, norm=dict(eps=1e-5), canon=dict(taps=3), layers=[
+        latent(4, 16, 16, 16, 48, dims=16, ff=64),
+        recurrent(64, 4, 4),
+        latent(20, 8, 16, 8, 112, dims=8, base=1000.0)]),
 }
-SEEDS = {"P": 11, "Q": 22, "R": 33}
+SEEDS = {"P": 11, "Q": 22, "R": 33, "S": 44}
 
 
 def tensors_for(config: dict, seed: int, query_factor: float = 3.0, sink_mean: float = 0.0) -> Dict[str, torch.Tensor]:
