@@ -236,17 +236,16 @@ int bc4g_xielu(const void* in, void* out, int dtype, const float* pq, long total
 int bc4g_causal_conv(const void* in, int dtype, const float* in_bias, const float* w, const float* out_bias, int add_input,
                      void* out, void* state, const int32_t* row_seq, const int32_t* seq_start, const int32_t* seq_slots,
                      int n_rows, int n_seqs, int channels, int taps, void* stream);
-// The gates of the real-gated linear recurrent unit: u [T, width] in `blocks` equal parts; ra_t, ri_t
-// [blocks][in][out] (the block matrices transposed); decay = exp(-8 sigmoid(Ra u + ra_b) softplus(lam)),
-// drive = sqrt(1 - decay^2) sigmoid(Ri u + ri_b) u, both float32 [T, width].
-int bc4g_rglru_gates(const void* u, int dtype, const void* ra_t, const void* ri_t, int w_dtype, const float* ra_b,
-                     const float* ri_b, const float* lam, float* decay, float* drive, int n_rows, int width, int blocks,
-                     void* stream);
-// S_t = decay_t S_(t-1) + drive_t along every request's rows, from state [slots, width] (float32) and back into it;
-// out[t] = S_t * gelu_tanh(y[t] + y_bias).
-int bc4g_rglru_scan(const float* decay, const float* drive, const void* y, int dtype, const float* y_bias, void* out,
-                    float* state, const int32_t* seq_start, const int32_t* seq_slots, int n_rows, int n_seqs, int width,
-                    void* stream);
+// The real-gated linear recurrent unit over a step's rows.  pre [T, blocks, 2 bs] (float32): the gates' sums of
+// every block, Ra u_b then Ri u_b (a product per block: bc4g_heads_gemm); u, y [T, width]; decay a = exp(-8
+// sigmoid(Ra u + ra_b) softplus(lam)), S_t = a S_(t-1) + sqrt(1 - a^2) sigmoid(Ri u + ri_b) u along every request's
+// rows, from state [slots, width] (float32) and back into it; out[t] = S_t * gelu_tanh(y[t] + y_bias).  A request's
+// rows are walked in chunks of 64 by threads of their own: chunk_a, chunk_b [S, ceil(most_rows / 64), width] and
+// before [S, width] are scratch (float32); most_rows: the most rows one request brings.
+int bc4g_rglru_scan(const float* pre, const void* u, const void* y, int dtype, const float* ra_b, const float* ri_b,
+                    const float* lam, const float* y_bias, void* out, float* state, float* chunk_a, float* chunk_b,
+                    float* before, const int32_t* seq_start, const int32_t* seq_slots, int n_rows, int n_seqs, int most_rows,
+                    int width, int blocks, void* stream);
 
 // Latent attention (attention_latent.hip).  q [T, heads, plain + rot] and dkv [T, rank + rot] as projected; the row's
 // cache slot (slot_map[t] = page * page_tokens + offset; cache [pages, page_tokens, rank + rot]; null: nothing is

@@ -15,6 +15,7 @@
 
 #include "api.h"
 #include "common.h"
+#include "mfma.h"
 
 namespace bc4g {
 namespace {
@@ -119,6 +120,58 @@ __global__ __launch_bounds__(256) void heads_gemm_kernel(const TA* __restrict__ 
       const int r = m0 + ty * 4 + i, c = n0 + tx * 4 + j;
       if (r < m && c < n) out[r * o_row + h * o_head + c] = from_float<TO>(acc[i][j]);
     }
+}
+
+// The same on the matrix cores for bfloat16 weights: a wave takes 16 rows x 16 NB columns of one head; both operands
+// have k side by side in memory, so a lane's eight k-slots are one load of 16 bytes (activations in float32 are
+// rounded to bfloat16 on the way); no LDS.  k a multiple of 8, every row and head of a on a 16-byte boundary.
+__device__ inline uint4 load_slots(const bf16_t* p) { return load16(p); }
+__device__ inline uint4 load_slots(const float* p) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  auto two = [](float lo, float hi) {
+    return static_cast<unsigned>(bf16_bits_from_float(lo)) | (static_cast<unsigned>(bf16_bits_from_float(hi)) << 16);
+  };
+  return make_uint4(two(a.x, a.y), two(a.z, a.w), two(b.x, b.y), two(b.z, b.w));
+}
+
+template <typename TA, typename TO, int NB>
+__global__ __launch_bounds__(kWave) void heads_mfma_kernel(const TA* __restrict__ a, long a_row, long a_head,
+                                                           const bf16_t* __restrict__ w, TO* __restrict__ out, long o_row,
+                                                           long o_head, int m, int n, int k) {
+  const int h = blockIdx.z, m0 = blockIdx.x * 16, n0 = blockIdx.y * 16 * NB;
+  const int c = threadIdx.x % 16, g = threadIdx.x / 16;
+  const bool row_there = m0 + c < m;
+  const TA* arow = a + (m0 + c) * a_row + h * a_head + 8 * g;
+  const bf16_t* wcol[NB];
+  bool col_there[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    col_there[nb] = n0 + nb * 16 + c < n;
+    wcol[nb] = w + (static_cast<long>(h) * n + n0 + nb * 16 + c) * k + 8 * g;
+  }
+  floatx4 acc[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) acc[nb] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int k0 = 0; k0 < k; k0 += 32) {
+    const bool k_there = k0 + 8 * g < k;
+    const uint4 av = row_there && k_there ? load_slots(arow + k0) : zero16();
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      const uint4 wv = col_there[nb] && k_there ? load16(wcol[nb] + k0) : zero16();
+      acc[nb] = mfma_16x16x32(av, wv, acc[nb]);
+    }
+  }
+  // a lane holds column c of every block and rows 4g .. 4g + 3
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    if (!col_there[nb]) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = m0 + 4 * g + i;
+      if (r < m) out[r * o_row + h * o_head + n0 + nb * 16 + c] = from_float<TO>(acc[nb][i]);
+    }
+  }
 }
 
 // ---- the attention ---------------------------------------------------------------------------------------------------
@@ -253,6 +306,24 @@ extern "C" int bc4g_heads_gemm(const void* a, int a_dtype, long a_row, long a_he
   BC4G_REQUIRE(ceil_div(n, kHT) <= 65535, "heads_gemm: n=%d is beyond the grid limit", n);
   if (m == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  // bfloat16 weights with k in whole pieces of 16 bytes: the matrix cores
+  const int a_bytes = a_dtype == kBF16 ? 2 : 4;
+  if (w_dtype == kBF16 && k % 8 == 0 && a_row % 8 == 0 && a_head % 8 == 0 && reinterpret_cast<uintptr_t>(a) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(w) % 16 == 0 && (a_bytes == 2 || a_dtype == kF32) && (out_dtype == kF32 || out_dtype == kBF16)) {
+    constexpr int kNB = 4;
+    dim3 mgrid(ceil_div(m, 16), ceil_div(n, 16 * kNB), heads);
+    BC4G_REQUIRE(mgrid.y <= 65535, "heads_gemm: n=%d is beyond the grid limit", n);
+    const bf16_t* wp = static_cast<const bf16_t*>(w);
+#define BC4G_HM(TA, TO)                                                                                                      \
+  heads_mfma_kernel<TA, TO, kNB><<<mgrid, kWave, 0, s>>>(static_cast<const TA*>(a), a_row, a_head, wp, static_cast<TO*>(out), \
+                                                         o_row, o_head, m, n, k)
+    if (a_dtype == kBF16 && out_dtype == kF32) BC4G_HM(bf16_t, float);
+    else if (a_dtype == kBF16) BC4G_HM(bf16_t, bf16_t);
+    else if (out_dtype == kF32) BC4G_HM(float, float);
+    else BC4G_HM(float, bf16_t);
+#undef BC4G_HM
+    return check_launch("heads_gemm");
+  }
   dim3 grid(ceil_div(m, kHT), ceil_div(n, kHT), heads);
 #define BC4G_HG(TA, TW, TO)                                                                                              \
   heads_gemm_kernel<TA, TW, TO><<<grid, 256, 0, s>>>(static_cast<const TA*>(a), a_row, a_head, static_cast<const TW*>(w), \

@@ -10,8 +10,10 @@
 //            holds, for its query, eight of the 32 keys, so maximum and sum of a query are in-lane plus two lane swaps
 //   output   O^T[latent x queries] += V^T[latent x keys] P^T[keys x queries] with V = the first `rank` numbers of the
 //            same LDS rows: the weights go from the score registers straight into the B operand (which key a k-slot
-//            stands for is free, as long as A agrees), and the A operand gathers its eight keys of one latent number
-//            from LDS two bytes at a time
+//            stands for is free, as long as A agrees); the A operand wants eight keys of one latent number side by
+//            side, so the latent part of a tile is kept a second time in LDS, transposed ([number][key]), written
+//            two bytes at a time while the tile is staged and read eight bytes at a time (gathering the keys from the
+//            rows themselves, two bytes a read, made the walk wait for LDS 256 times a tile)
 //
 // The keys may be cut into n_splits parts over workgroups (few rows over a long context: a decode step), whose
 // unnormalised float partials a second kernel merges; the sink joins the sum where the sum is finished.
@@ -26,6 +28,7 @@ namespace bc4g {
 namespace {
 
 constexpr int kKeys = 32;                   // cache rows a key tile holds
+constexpr int kVtPitch = 36;                // 16-bit elements of a row of the transposed latent part (32 keys and a pad)
 constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ inline unsigned pack_bf16(float lo, float hi) {
@@ -34,16 +37,18 @@ __device__ inline unsigned pack_bf16(float lo, float hi) {
 
 // KS: k-steps of 32 over a cache row (dk <= 32 KS); DB: blocks of 16 over the latent (rank <= 16 DB).
 template <int KS, int DB>
-__global__ __launch_bounds__(256) void latent_mfma_kernel(
+__global__ __launch_bounds__(256, 2) void latent_mfma_kernel(
     const float* __restrict__ q_lat, float* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     const bf16_t* __restrict__ cache, const float* __restrict__ sink, const int32_t* __restrict__ block_table,
     int table_stride, const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_ctx, int n_tokens, int heads,
     int rank, int dk, int page_tokens, int window, float scale, int hb, int tpt, int n_hg, int n_splits) {
-  extern __shared__ uint4 tile[];                             // [kKeys][dk / 8 + 1] pieces of 16 bytes
+  extern __shared__ uint4 tile[];                             // [kKeys][dk / 8 + 1] pieces of 16 bytes, then the transposed part
   const int s = blockIdx.y, z = blockIdx.z;
   const int tok0 = seq_start[s], n_tok = seq_start[s + 1] - tok0, cached = seq_ctx[s];
   const int n_tb = (n_tok + tpt - 1) / tpt, n_tiles = n_tb * n_hg;
-  const int tile0 = blockIdx.x * 4;
+  // (the grid's first workgroups take a request's last rows: their walks over the keys are the longest, and the short
+  // ones fill in behind them)
+  const int tile0 = (gridDim.x - 1 - blockIdx.x) * 4;
   if (tile0 >= n_tiles) return;                               // (the whole workgroup)
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int my_tile = tile0 + wave;
@@ -82,24 +87,44 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
   for (int db = 0; db < DB; ++db) acc[db] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
   const float scale2 = scale * kLog2e;                        // exponents to the base 2
-  const uint16_t* tile16 = reinterpret_cast<const uint16_t*>(tile);
-  const int pitch16 = pitch * 8;
+  uint16_t* vt = reinterpret_cast<uint16_t*>(tile + kKeys * pitch);     // [rank][kVtPitch]: the latent part, transposed
 
+  // Staging: eight threads a key, each with every eighth 16-byte piece of its row -- one look at the block table a
+  // thread and tile, all of a thread's loads asked for together, and the next tile's asked for before this tile is
+  // worked on, so that they are under way meanwhile (the barriers wait for LDS only).
+  constexpr int kPieces = (KS * 4 + 7) / 8;
+  const int st_key = threadIdx.x / 8, st_sub = threadIdx.x % 8;
+  uint4 stage[kPieces];
+  auto fetch = [&](int kt) {
+    const int j = kt * kKeys + st_key;
+    const bool there = j >= first_pos && j <= last_pos;
+    const bf16_t* src = cache;
+    if (there) src = cache + (static_cast<long>(table[j / page_tokens]) * page_tokens + j % page_tokens) * dk;
+#pragma unroll
+    for (int p = 0; p < kPieces; ++p) {
+      const int part = st_sub + 8 * p;
+      stage[p] = there && part < cpr ? load16(src + part * 8) : zero16();
+    }
+  };
   for (int kt = kt_lo; kt < kt_hi; ++kt) {
     const int j0 = kt * kKeys;
-    __syncthreads();                                          // the tile before has been read by everyone
-    for (int piece = threadIdx.x; piece < kKeys * cpr; piece += 256) {
-      const int key = piece / cpr, part = piece - key * cpr;
-      const int j = j0 + key;
-      uint4 v = zero16();
-      if (j >= first_pos && j <= last_pos) {
-        const long page = table[j / page_tokens];
-        v = load16(cache + (page * page_tokens + j % page_tokens) * dk + part * 8);
+    fetch(kt);
+#pragma unroll
+    for (int p = 0; p < kPieces; ++p) {
+      const int part = st_sub + 8 * p;
+      if (part < cpr) tile[st_key * pitch + part] = stage[p];
+      if (part * 8 < rank) {
+        uint16_t* to = vt + part * 8 * kVtPitch + st_key;
+        const unsigned w[4] = {stage[p].x, stage[p].y, stage[p].z, stage[p].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          to[(2 * e) * kVtPitch] = static_cast<uint16_t>(w[e] & 0xffffu);
+          to[(2 * e + 1) * kVtPitch] = static_cast<uint16_t>(w[e] >> 16);
+        }
       }
-      tile[key * pitch + part] = v;
     }
-    __syncthreads();
-    if (!wave_live) continue;
+    lds_barrier();
+    if (wave_live) {
     floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -135,18 +160,18 @@ __global__ __launch_bounds__(256) void latent_mfma_kernel(
       for (int db = 0; db < DB; ++db) acc[db] *= alpha;
     }
     const uint4 pf = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
-    const uint16_t* col = tile16 + (4 * g) * pitch16 + c;     // key 4g, latent number c of a block
+    const uint16_t* col = vt + c * kVtPitch + 4 * g;          // latent number c of a block, keys 4g .. 4g + 3
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
       if (db * 16 < rank) {
-        const uint16_t* v = col + db * 16;
-        const uint4 a = make_uint4(
-            v[0] | (static_cast<unsigned>(v[pitch16]) << 16), v[2 * pitch16] | (static_cast<unsigned>(v[3 * pitch16]) << 16),
-            v[16 * pitch16] | (static_cast<unsigned>(v[17 * pitch16]) << 16),
-            v[18 * pitch16] | (static_cast<unsigned>(v[19 * pitch16]) << 16));
+        const uint2 lo = *reinterpret_cast<const uint2*>(col + db * 16 * kVtPitch);
+        const uint2 hi = *reinterpret_cast<const uint2*>(col + db * 16 * kVtPitch + 16);
+        const uint4 a = make_uint4(lo.x, lo.y, hi.x, hi.y);
         acc[db] = mfma_16x16x32(a, pf, acc[db]);
       }
     }
+    }
+    lds_barrier();                                            // the tile has been read by everyone
   }
   if (!q_live) return;
   l += __shfl_xor(l, 16, kWave);
@@ -179,18 +204,21 @@ __global__ __launch_bounds__(kWave) void latent_merge_kernel(const float* __rest
                                                              const float* __restrict__ sink, float* __restrict__ out,
                                                              long rows, int heads, int rank, int n_splits) {
   const long row = blockIdx.x;
-  float big = -INFINITY;
-  for (int z = 0; z < n_splits; ++z) big = fmaxf(big, part_ml[(z * rows + row) * 2]);
-  float total = sink ? __builtin_amdgcn_exp2f(sink[row % heads] * kLog2e - big) : 0.f;
-  for (int z = 0; z < n_splits; ++z) {
-    const float* ml = part_ml + (z * rows + row) * 2;
-    total += ml[1] * __builtin_amdgcn_exp2f(ml[0] - big);
+  const int lane = threadIdx.x;
+  // a lane a part for the maxima and sums (at most 64 parts), then a lane a number of the latent
+  float mz = -INFINITY, lz = 0.f;
+  if (lane < n_splits) {
+    const float2 ml = *reinterpret_cast<const float2*>(part_ml + (lane * rows + row) * 2);
+    mz = ml.x, lz = ml.y;
   }
+  const float big = wave_max(mz);
+  const float wz = __builtin_amdgcn_exp2f(mz - big);
+  const float total = wave_sum(lz * wz) + (sink ? __builtin_amdgcn_exp2f(sink[row % heads] * kLog2e - big) : 0.f);
   const float inv = 1.0f / total;
-  for (int d = threadIdx.x; d < rank; d += kWave) {
+  for (int d = lane; d < rank; d += kWave) {
     float sum = 0.f;
-    for (int z = 0; z < n_splits; ++z)
-      sum += part_o[(z * rows + row) * rank + d] * __builtin_amdgcn_exp2f(part_ml[(z * rows + row) * 2] - big);
+#pragma unroll 4
+    for (int z = 0; z < n_splits; ++z) sum = fmaf(part_o[(z * rows + row) * rank + d], __shfl(wz, z, kWave), sum);
     out[row * rank + d] = sum * inv;
   }
 }
@@ -231,15 +259,20 @@ extern "C" int bc4g_attention_latent_mfma(const float* q_lat, float* out, float*
   const int most_tiles = ceil_div(most_tokens, tpt) * n_hg;
   BC4G_REQUIRE(n_seqs <= 65535 && n_splits <= 65535, "attention_latent_mfma: %d requests are beyond the grid limit", n_seqs);
   dim3 grid(ceil_div(most_tiles, 4), n_seqs, n_splits);
-  const size_t lds = static_cast<size_t>(kKeys) * (dk / 8 + 1) * 16;
+  const size_t lds = static_cast<size_t>(kKeys) * (dk / 8 + 1) * 16 + static_cast<size_t>(rank) * kVtPitch * 2;
   const bf16_t* kc = static_cast<const bf16_t*>(cache);
+  // (more than 64 KB of LDS a workgroup has to be asked for, once for a kernel: the most this kernel ever takes)
 #define BC4G_LATENT(KS, DB)                                                                                                 \
+  static const hipError_t allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_mfma_kernel<KS, DB>),         \
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize,                          \
+                                                        kKeys * (KS * 4 + 1) * 16 + DB * 16 * kVtPitch * 2);                 \
+  BC4G_REQUIRE(allowed == hipSuccess, "attention_latent_mfma: %zu bytes of LDS a workgroup are refused", lds);              \
   latent_mfma_kernel<KS, DB><<<grid, 256, lds, s>>>(q_lat, out, part_o, part_ml, kc, sink, block_table, table_stride, seq_start, \
                                                     seq_ctx, n_tokens, heads, rank, dk, page_tokens, window, scale, hb, tpt, n_hg, \
                                                     n_splits)
-  if (dk <= 128 && rank <= 64) BC4G_LATENT(4, 4);
-  else if (dk <= 320 && rank <= 256) BC4G_LATENT(10, 16);
-  else BC4G_LATENT(18, 32);
+  if (dk <= 128 && rank <= 64) { BC4G_LATENT(4, 4); }
+  else if (dk <= 320 && rank <= 256) { BC4G_LATENT(10, 16); }
+  else { BC4G_LATENT(18, 32); }
 #undef BC4G_LATENT
   if (n_splits > 1)
     latent_merge_kernel<<<static_cast<unsigned>(static_cast<long>(n_tokens) * heads), kWave, 0, s>>>(

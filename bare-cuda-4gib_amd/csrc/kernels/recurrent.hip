@@ -81,79 +81,59 @@ __device__ inline float gelu_tanh_f(float z) {
   return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
 
-constexpr int kGateRows = 16;      // rows of a workgroup: four a wave
-constexpr int kGateChunk = 64;     // inputs staged in LDS at a time
+constexpr int kChunk = 64;         // rows of a request that one thread walks
 
-// The gates of the recurrence, for channel ch of block b = ch / bs:  r = sigmoid(Ra[b] u_b + ra_b), i = sigmoid(Ri[b] u_b
-// + ri_b); decay[t, ch] = a = exp(-8 r softplus(lam)); drive[t, ch] = sqrt(1 - a^2) i u.  The block matrices come
-// transposed, [block][in][out], so that a wave's lanes (one output each) read side by side.  Sums over the inputs
-// in ascending order in one thread.
-template <typename T, typename TW>
-__global__ __launch_bounds__(kBlock) void rglru_gates_kernel(const T* __restrict__ u, const TW* __restrict__ ra_t,
-                                                             const TW* __restrict__ ri_t, const float* __restrict__ ra_b,
-                                                             const float* __restrict__ ri_b, const float* __restrict__ lam,
-                                                             float* __restrict__ decay, float* __restrict__ drive,
-                                                             int n_rows, int width, int bs) {
-  __shared__ float u_s[kGateRows][kGateChunk];
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int row0 = blockIdx.x * kGateRows, b = blockIdx.y, o = blockIdx.z * kWave + lane;
-  const TW* wa = ra_t + static_cast<long>(b) * bs * bs;
-  const TW* wi = ri_t + static_cast<long>(b) * bs * bs;
-  float sa[4] = {0.f, 0.f, 0.f, 0.f}, si[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < bs; k0 += kGateChunk) {
-    const int kn = min(kGateChunk, bs - k0);
-    for (int e = threadIdx.x; e < kGateRows * kGateChunk; e += kBlock) {
-      const int r = e / kGateChunk, k = e % kGateChunk;
-      const int row = row0 + r;
-      u_s[r][k] = (row < n_rows && k < kn) ? to_float(u[static_cast<long>(row) * width + b * bs + k0 + k]) : 0.f;
-    }
-    __syncthreads();
-    if (o < bs) {
-      for (int k = 0; k < kn; ++k) {
-        const float a = to_float(wa[static_cast<long>(k0 + k) * bs + o]), i = to_float(wi[static_cast<long>(k0 + k) * bs + o]);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float uv = u_s[wave * 4 + r][k];
-          sa[r] = fmaf(a, uv, sa[r]);
-          si[r] = fmaf(i, uv, si[r]);
-        }
-      }
-    }
-    __syncthreads();
-  }
-  if (o >= bs) return;
-  const int ch = b * bs + o;
-  const float sp = softplus_f(lam[ch]), ba = ra_b[ch], bi = ri_b[ch];
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int row = row0 + wave * 4 + r;
-    if (row >= n_rows) continue;
-    const float gate_r = sigmoid_f(sa[r] + ba), gate_i = sigmoid_f(si[r] + bi);
-    const float log_a = -8.0f * gate_r * sp;
-    const long at = static_cast<long>(row) * width + ch;
-    decay[at] = expf(log_a);
-    drive[at] = sqrtf(-expm1f(2.0f * log_a)) * gate_i * to_float(u[at]);
-  }
+// Decay and drive of one row and channel from the gates' sums: r = sigmoid(sum_a + ba), i = sigmoid(sum_i + bi),
+// a = exp(-8 r softplus(lam)), drive = sqrt(1 - a^2) i u  (1 - a^2 as -expm1(2 log a): exact also where a is close to 1).
+__device__ inline void decay_and_drive(float sum_a, float sum_i, float u, float ba, float bi, float sp, float* a, float* x) {
+  const float log_a = -8.0f * sigmoid_f(sum_a + ba) * sp;
+  *a = expf(log_a);
+  *x = sqrtf(-expm1f(2.0f * log_a)) * sigmoid_f(sum_i + bi) * u;
 }
 
-// S_t = decay_t S_(t-1) + drive_t along a request's rows, from the request's state and back into it;
-// out[t] = S_t * gelu_tanh(y[t] + y_bias).  A thread takes one (request, channel).
-template <typename T>
-__global__ void rglru_scan_kernel(const float* __restrict__ decay, const float* __restrict__ drive, const T* __restrict__ y,
-                                  const float* __restrict__ y_bias, T* __restrict__ out, float* __restrict__ state,
-                                  const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slots, int width) {
-  const int ch = blockIdx.x * blockDim.x + threadIdx.x, s = blockIdx.y;
-  if (ch >= width) return;
+// The recurrence S_t = a_t S_(t-1) + x_t over a request's rows in chunks of kChunk, so that a long prompt's rows are
+// walked by many threads: a thread takes (channel, chunk, request).  First pass: what the chunk does to a state,
+// S_out = A S_in + B; the first chunk's thread also notes the request's state before the step.  Second pass: the
+// state before the chunk from the chunks before it, then the chunk's rows for good: out[t] = S_t gelu_tanh(y[t] + by);
+// the last chunk's thread leaves the state.  pre [T, blocks, 2 bs] holds the gates' sums (Ra u, then Ri u, of a block).
+template <typename T, bool kSecond>
+__global__ __launch_bounds__(kWave) void rglru_chunks_kernel(
+    const float* __restrict__ pre, const T* __restrict__ u, const T* __restrict__ y, const float* __restrict__ ra_b,
+    const float* __restrict__ ri_b, const float* __restrict__ lam, const float* __restrict__ y_bias, T* __restrict__ out,
+    float* __restrict__ state, float* __restrict__ chunk_a, float* __restrict__ chunk_b, float* __restrict__ before,
+    const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slots, int width, int bs, int most_chunks) {
+  const int ch = blockIdx.x * kWave + threadIdx.x, chunk = blockIdx.y, s = blockIdx.z;
   const long start = seq_start[s], end = seq_start[s + 1];
+  const long lo = start + static_cast<long>(chunk) * kChunk, hi = lo + kChunk < end ? lo + kChunk : end;
+  if (ch >= width || lo >= end) return;
+  const int b = ch / bs, o = ch - b * bs;
+  const float ba = ra_b[ch], bi = ri_b[ch], sp = softplus_f(lam[ch]);
+  const float* pa = pre + static_cast<long>(b) * 2 * bs + o;           // + t * 2 * width; the other gate bs further
   float* slot = state + static_cast<long>(seq_slots[s]) * width + ch;
-  const float yb = y_bias ? y_bias[ch] : 0.f;
-  float st = *slot;
-  for (long t = start; t < end; ++t) {
-    const long at = t * width + ch;
-    st = fmaf(decay[at], st, drive[at]);
-    out[at] = from_float<T>(st * gelu_tanh_f(to_float(y[at]) + yb));
+  const long note = (static_cast<long>(s) * most_chunks) * width + ch;   // + chunk * width
+  if (!kSecond) {
+    float A = 1.f, B = 0.f;
+    for (long t = lo; t < hi; ++t) {
+      float a, x;
+      decay_and_drive(pa[t * 2 * width], pa[t * 2 * width + bs], to_float(u[t * width + ch]), ba, bi, sp, &a, &x);
+      B = fmaf(a, B, x);
+      A *= a;
+    }
+    chunk_a[note + static_cast<long>(chunk) * width] = A;
+    chunk_b[note + static_cast<long>(chunk) * width] = B;
+    if (chunk == 0) before[static_cast<long>(s) * width + ch] = *slot;
+  } else {
+    float st = before[static_cast<long>(s) * width + ch];
+    for (int c = 0; c < chunk; ++c) st = fmaf(chunk_a[note + static_cast<long>(c) * width], st, chunk_b[note + static_cast<long>(c) * width]);
+    const float yb = y_bias ? y_bias[ch] : 0.f;
+    for (long t = lo; t < hi; ++t) {
+      float a, x;
+      decay_and_drive(pa[t * 2 * width], pa[t * 2 * width + bs], to_float(u[t * width + ch]), ba, bi, sp, &a, &x);
+      st = fmaf(a, st, x);
+      out[t * width + ch] = from_float<T>(st * gelu_tanh_f(to_float(y[t * width + ch]) + yb));
+    }
+    if (hi == end) *slot = st;
   }
-  *slot = st;
 }
 
 }  // namespace
@@ -188,45 +168,31 @@ extern "C" int bc4g_causal_conv(const void* in, int dtype, const float* in_bias,
   return check_launch("causal_conv");
 }
 
-extern "C" int bc4g_rglru_gates(const void* u, int dtype, const void* ra_t, const void* ri_t, int w_dtype, const float* ra_b,
-                                const float* ri_b, const float* lam, float* decay, float* drive, int n_rows, int width,
-                                int blocks, void* stream) {
-  BC4G_REQUIRE(n_rows >= 0 && width > 0 && blocks > 0 && width % blocks == 0, "rglru_gates: bad sizes T=%d W=%d blocks=%d",
-               n_rows, width, blocks);
-  BC4G_REQUIRE(u && ra_t && ri_t && ra_b && ri_b && lam && decay && drive, "rglru_gates: a tensor is missing");
-  BC4G_REQUIRE(blocks <= 65535, "rglru_gates: %d blocks are beyond the grid limit", blocks);
-  if (n_rows == 0) return 0;
+extern "C" int bc4g_rglru_scan(const float* pre, const void* u, const void* y, int dtype, const float* ra_b, const float* ri_b,
+                               const float* lam, const float* y_bias, void* out, float* state, float* chunk_a, float* chunk_b,
+                               float* before, const int32_t* seq_start, const int32_t* seq_slots, int n_rows, int n_seqs,
+                               int most_rows, int width, int blocks, void* stream) {
+  BC4G_REQUIRE(n_rows >= 0 && n_seqs >= 0 && width > 0 && blocks > 0 && width % blocks == 0 && n_seqs <= 65535 && most_rows >= 0,
+               "rglru_scan: bad sizes T=%d S=%d W=%d blocks=%d", n_rows, n_seqs, width, blocks);
+  BC4G_REQUIRE(pre && u && y && ra_b && ri_b && lam && out && state && chunk_a && chunk_b && before && seq_start && seq_slots,
+               "rglru_scan: a tensor is missing");
+  if (n_rows == 0 || n_seqs == 0 || most_rows == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int bs = width / blocks;
-  dim3 grid(ceil_div(n_rows, kGateRows), blocks, ceil_div(bs, kWave));
-#define BC4G_GATES(T, TW)                                                                                            \
-  rglru_gates_kernel<T, TW><<<grid, kBlock, 0, s>>>(static_cast<const T*>(u), static_cast<const TW*>(ra_t),         \
-                                                    static_cast<const TW*>(ri_t), ra_b, ri_b, lam, decay, drive,    \
-                                                    n_rows, width, bs)
-  if (dtype == kF32 && w_dtype == kF32) BC4G_GATES(float, float);
-  else if (dtype == kBF16 && w_dtype == kBF16) BC4G_GATES(bf16_t, bf16_t);
-  else if (dtype == kBF16 && w_dtype == kF32) BC4G_GATES(bf16_t, float);
-  else if (dtype == kF32 && w_dtype == kBF16) BC4G_GATES(float, bf16_t);
-  else return fail("rglru_gates: unknown dtypes %d, %d", dtype, w_dtype);
-#undef BC4G_GATES
-  return check_launch("rglru_gates");
-}
-
-extern "C" int bc4g_rglru_scan(const float* decay, const float* drive, const void* y, int dtype, const float* y_bias, void* out,
-                               float* state, const int32_t* seq_start, const int32_t* seq_slots, int n_rows, int n_seqs,
-                               int width, void* stream) {
-  BC4G_REQUIRE(n_rows >= 0 && n_seqs >= 0 && width > 0 && n_seqs <= 65535, "rglru_scan: bad sizes T=%d S=%d W=%d", n_rows,
-               n_seqs, width);
-  BC4G_REQUIRE(decay && drive && y && out && state && seq_start && seq_slots, "rglru_scan: a tensor is missing");
-  if (n_rows == 0 || n_seqs == 0) return 0;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  dim3 grid(ceil_div(width, kWave), n_seqs);
-  if (dtype == kF32)
-    rglru_scan_kernel<float><<<grid, kWave, 0, s>>>(decay, drive, static_cast<const float*>(y), y_bias,
-                                                    static_cast<float*>(out), state, seq_start, seq_slots, width);
-  else if (dtype == kBF16)
-    rglru_scan_kernel<bf16_t><<<grid, kWave, 0, s>>>(decay, drive, static_cast<const bf16_t*>(y), y_bias,
-                                                     static_cast<bf16_t*>(out), state, seq_start, seq_slots, width);
+  const int most_chunks = ceil_div(most_rows, kChunk);
+  BC4G_REQUIRE(most_chunks <= 65535, "rglru_scan: %d rows of one request are beyond the grid limit", most_rows);
+  dim3 grid(ceil_div(width, kWave), most_chunks, n_seqs);
+#define BC4G_SCAN(T)                                                                                                            \
+  do {                                                                                                                          \
+    rglru_chunks_kernel<T, false><<<grid, kWave, 0, s>>>(pre, static_cast<const T*>(u), static_cast<const T*>(y), ra_b, ri_b,  \
+                                                         lam, y_bias, static_cast<T*>(out), state, chunk_a, chunk_b, before,   \
+                                                         seq_start, seq_slots, width, width / blocks, most_chunks);            \
+    rglru_chunks_kernel<T, true><<<grid, kWave, 0, s>>>(pre, static_cast<const T*>(u), static_cast<const T*>(y), ra_b, ri_b,   \
+                                                        lam, y_bias, static_cast<T*>(out), state, chunk_a, chunk_b, before,    \
+                                                        seq_start, seq_slots, width, width / blocks, most_chunks);             \
+  } while (0)
+  if (dtype == kF32) BC4G_SCAN(float);
+  else if (dtype == kBF16) BC4G_SCAN(bf16_t);
   else return fail("rglru_scan: unknown dtype %d", dtype);
+#undef BC4G_SCAN
   return check_launch("rglru_scan");
 }

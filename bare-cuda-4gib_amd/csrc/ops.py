@@ -1210,33 +1210,37 @@ def causal_conv(x: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Ten
     return out
 
 
-def rglru(u: torch.Tensor, y: torch.Tensor, ra_t: torch.Tensor, ri_t: torch.Tensor, ra_b: torch.Tensor, ri_b: torch.Tensor,
+RGLRU_CHUNK = 64            # rows of a request that one thread of the recurrence walks
+
+
+def rglru(u: torch.Tensor, y: torch.Tensor, w_gates: torch.Tensor, ra_b: torch.Tensor, ri_b: torch.Tensor,
           lam: torch.Tensor, y_bias: Optional[torch.Tensor], state: torch.Tensor, ctx) -> torch.Tensor:
-    """The real-gated linear recurrent unit over a step's rows: u, y [T, W]; ra_t, ri_t [blocks, in, out] (the gates'
-    block matrices, transposed); biases and lam float32 [W]; state float32 [slots, W].  Gates, decay and state in
+    """The real-gated linear recurrent unit over a step's rows: u, y [T, W]; w_gates [blocks, 2 bs, bs] (of every block
+    the matrix of the recurrence gate, then that of the input gate, each [out, in]); biases and lam float32 [W]; state
+    float32 [slots, W].  The gates' sums are a product per block (float32 out), the gates, the decay and the state
     float32.  Returns S_t * gelu_tanh(y + y_bias) in u's dtype."""
-    _dev("rglru", u, y, ra_t, ri_t, ra_b, ri_b, lam, y_bias, state)
+    _dev("rglru", u, y, w_gates, ra_b, ri_b, lam, y_bias, state)
     if u.dim() != 2 or y.shape != u.shape or y.dtype != u.dtype:
         raise KernelError(f"rglru: u and y must be alike [T, W], got {tuple(u.shape)} and {tuple(y.shape)}")
     t, w = u.shape
-    if ra_t.dim() != 3 or ra_t.shape != ri_t.shape or ra_t.dtype != ri_t.dtype or ra_t.shape[1] != ra_t.shape[2] \
-            or ra_t.shape[0] * ra_t.shape[1] != w:
-        raise KernelError(f"rglru: gate matrices {tuple(ra_t.shape)}, {tuple(ri_t.shape)} do not cut {w} channels into square blocks")
+    if w_gates.dim() != 3 or w_gates.shape[1] != 2 * w_gates.shape[2] or w_gates.shape[0] * w_gates.shape[2] != w:
+        raise KernelError(f"rglru: gate matrices {tuple(w_gates.shape)} do not cut {w} channels into blocks of [2 bs, bs]")
     for name, v in (("ra_b", ra_b), ("ri_b", ri_b), ("lam", lam), ("y_bias", y_bias)):
         _f32("rglru", name, v, (w,))
     if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] != w or max(ctx.seq_slots, default=0) >= state.shape[0]:
         raise KernelError(f"rglru: state must be float32 [slots, {w}] with a row for every slot of the step")
     _check_grouping("rglru", ctx, t)
-    blocks, bs = ra_t.shape[0], ra_t.shape[1]
-    decay = torch.empty((t, w), dtype=torch.float32, device=u.device)
-    drive = torch.empty((t, w), dtype=torch.float32, device=u.device)
-    library.call("bc4g_rglru_gates", _ptr(u), _code(u, "rglru"), _ptr(ra_t), _ptr(ri_t), _code(ra_t, "rglru"), _ptr(ra_b),
-                 _ptr(ri_b), _ptr(lam), _ptr(decay), _ptr(drive), t, w, blocks, _stream(),
-                 cost=lambda: (4.0 * t * w * bs, 2 * w * bs * ra_t.element_size() + t * w * (u.element_size() + 8)))
+    blocks, bs = w_gates.shape[0], w_gates.shape[2]
+    pre = torch.empty((t, blocks, 2 * bs), dtype=torch.float32, device=u.device)
+    heads_gemm(u.view(t, blocks, bs), w_gates, pre, k=bs, n=2 * bs)
+    most = max(int(ctx.seq_start[s + 1] - ctx.seq_start[s]) for s in range(ctx.n_seqs))
+    chunks = -(-most // RGLRU_CHUNK)
+    scratch = torch.empty((2 * chunks + 1, ctx.n_seqs, w), dtype=torch.float32, device=u.device)
     out = torch.empty_like(u)
-    library.call("bc4g_rglru_scan", _ptr(decay), _ptr(drive), _ptr(y), _code(y, "rglru"), _ptr(y_bias), _ptr(out), _ptr(state),
-                 _ptr(ctx.seq_start_dev), _ptr(ctx.seq_slots_dev), t, ctx.n_seqs, w, _stream(),
-                 cost=lambda: (12.0 * t * w, t * w * (8 + 2 * u.element_size())))
+    library.call("bc4g_rglru_scan", _ptr(pre), _ptr(u), _ptr(y), _code(y, "rglru"), _ptr(ra_b), _ptr(ri_b), _ptr(lam), _ptr(y_bias),
+                 _ptr(out), _ptr(state), _ptr(scratch[:chunks]), _ptr(scratch[chunks:2 * chunks]), _ptr(scratch[2 * chunks]),
+                 _ptr(ctx.seq_start_dev), _ptr(ctx.seq_slots_dev), t, ctx.n_seqs, most, w, blocks, _stream(),
+                 cost=lambda: (40.0 * t * w, t * w * (16 + 5 * u.element_size())))
     return out
 
 
@@ -1257,14 +1261,14 @@ def attention_latent_mfma_takes(cache: torch.Tensor, rank: int, rot: int) -> boo
 def latent_splits(seq_start, heads: int, max_kv_len: int) -> int:
     """Into how many parts the matrix-core kernel cuts every walk over the keys: one where the step's rows fill the
     GPU by themselves (a workgroup takes four tiles of 16 (token, head) pairs of one request), else as many as bring
-    the workgroups to twice that, while a part keeps two key tiles of 32."""
+    the workgroups to twice that, while a part keeps a key tile of 32."""
     hb = min(heads, 16)
     tpt, n_hg = 16 // hb, -(-heads // hb)
     groups = sum(-(-(-(-int(seq_start[s + 1] - seq_start[s]) // tpt) * n_hg) // 4) for s in range(len(seq_start) - 1))
     if groups >= LATENT_ENOUGH_GROUPS or groups == 0:
         return 1
     key_tiles = -(-max_kv_len // 32)
-    return max(1, min(-(-2 * LATENT_ENOUGH_GROUPS // groups), key_tiles // 2, LATENT_MAX_SPLITS))
+    return max(1, min(-(-2 * LATENT_ENOUGH_GROUPS // groups), key_tiles, LATENT_MAX_SPLITS))
 
 
 def latent_prepare(q: torch.Tensor, dkv: torch.Tensor, g: torch.Tensor, eps: float, positions: torch.Tensor,

@@ -45,9 +45,8 @@ class RGLRU(Part):
         self.y_b, self.x_b, self.conv_b, self.lam = f32("y.b"), f32("x.b"), f32("conv.b"), f32("lam")
         self.ra_b, self.ri_b = f32("ra.b"), f32("ri.b")
         self.conv_w = tensors["conv"].to(torch.float32).contiguous()
-        # [block, in, out]: a wave's lanes, one output each, read side by side
-        self.ra_t = tensors["ra"].transpose(1, 2).contiguous()
-        self.ri_t = tensors["ri"].transpose(1, 2).contiguous()
+        # [block, 2 bs, bs]: both gates' matrices of a block in one product per block
+        self.w_gates = torch.cat([tensors["ra"], tensors["ri"]], dim=1).contiguous()
         self.act_dtype = rt.act_dtype
 
     def forward(self, h, ctx, cache, residual, writes: bool = True) -> None:
@@ -55,7 +54,7 @@ class RGLRU(Part):
         x = linear(h, self.w_x, out_dtype=self.act_dtype)
         u = ops.causal_conv(x, self.conv_w, cache.tail if self.conv_taps > 1 else None, ctx, in_bias=self.x_b,
                             out_bias=self.conv_b)
-        out = ops.rglru(u, y, self.ra_t, self.ri_t, self.ra_b, self.ri_b, self.lam, self.y_b, cache.state, ctx)
+        out = ops.rglru(u, y, self.w_gates, self.ra_b, self.ri_b, self.lam, self.y_b, cache.state, ctx)
         linear(out, self.w_o, accumulate_into=residual, ctx=ctx)
 
 

@@ -278,7 +278,7 @@ def test_recurrence_over_portions(dtype, blocks, width):
     (large lam) and close to zero both occur."""
     from bare_cuda_4gib_amd.csrc import ops
     torch.manual_seed(width)
-    dev, T, bs = "cuda:0", 150, width // blocks
+    dev, T, bs = "cuda:0", 350, width // blocks
     u, y = torch.randn(T, width).to(dtype), torch.randn(T, width).to(dtype)
     ra, ri = (torch.randn(blocks, bs, bs) / math.sqrt(bs)).to(dtype), (torch.randn(blocks, bs, bs) / math.sqrt(bs)).to(dtype)
     ra_b, ri_b, lam, y_b = torch.randn(width), torch.randn(width), torch.randn(width) * 3 - 2, torch.randn(width) * 0.3
@@ -294,10 +294,9 @@ def test_recurrence_over_portions(dtype, blocks, width):
     state = torch.full((3, width), 9.0, device=dev)
     state[1].zero_()
     got, at = [], 0
-    for n in (1, 2, 40, 1, 1, 64, 3, 38):
+    for n in (1, 2, 40, 1, 1, 64, 3, 38, 200):
         ctx = step_context([n], [at], [1])
-        got.append(ops.rglru(u[at:at + n].to(dev), y[at:at + n].to(dev), ra.transpose(1, 2).contiguous().to(dev),
-                             ri.transpose(1, 2).contiguous().to(dev), ra_b.to(dev), ri_b.to(dev), lam.to(dev), y_b.to(dev), state, ctx).cpu())
+        got.append(ops.rglru(u[at:at + n].to(dev), y[at:at + n].to(dev), torch.cat([ra, ri], dim=1).contiguous().to(dev), ra_b.to(dev), ri_b.to(dev), lam.to(dev), y_b.to(dev), state, ctx).cpu())
         at += n
     tol = 2e-5 if dtype == torch.float32 else 2e-2
     assert torch.allclose(torch.cat(got).double(), want, atol=tol, rtol=tol)
