@@ -152,7 +152,7 @@ __global__ __launch_bounds__(kWave) void heads_mfma_kernel(const TA* __restrict_
   floatx4 acc[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) acc[nb] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
+#pragma unroll 8
   for (int k0 = 0; k0 < k; k0 += 32) {
     const bool k_there = k0 + 8 * g < k;
     const uint4 av = row_there && k_there ? load_slots(arow + k0) : zero16();
@@ -180,7 +180,7 @@ __global__ __launch_bounds__(kWave) void heads_mfma_kernel(const TA* __restrict_
 // the scores (lane = key, the sum over the numbers in ascending order), then, once the tile's weights are known, its
 // latent part again for the output (lane = number, the sum over the keys in ascending order).  Keys are walked in
 // ascending order from the first the row sees, with a running maximum and sum; the sink joins the sum at the end.
-constexpr int kMaxLatentRow = 640;                    // rank + rot at most
+constexpr int kMaxLatentRow = 1024;                   // rank + rot at most
 constexpr int kLatentChunks = kMaxLatentRow / kWave;
 constexpr int kHeadsPerGroup = 8;
 constexpr int kTilePad = kWave + 1;
@@ -310,13 +310,20 @@ extern "C" int bc4g_heads_gemm(const void* a, int a_dtype, long a_row, long a_he
   const int a_bytes = a_dtype == kBF16 ? 2 : 4;
   if (w_dtype == kBF16 && k % 8 == 0 && a_row % 8 == 0 && a_head % 8 == 0 && reinterpret_cast<uintptr_t>(a) % 16 == 0 &&
       reinterpret_cast<uintptr_t>(w) % 16 == 0 && (a_bytes == 2 || a_dtype == kF32) && (out_dtype == kF32 || out_dtype == kBF16)) {
-    constexpr int kNB = 4;
-    dim3 mgrid(ceil_div(m, 16), ceil_div(n, 16 * kNB), heads);
+    // few rows (a decode step): a wave takes one block of 16 columns, so that more waves share the weights' way in
+    const int nb = m <= 32 ? 1 : 4;
+    dim3 mgrid(ceil_div(m, 16), ceil_div(n, 16 * nb), heads);
     BC4G_REQUIRE(mgrid.y <= 65535, "heads_gemm: n=%d is beyond the grid limit", n);
     const bf16_t* wp = static_cast<const bf16_t*>(w);
-#define BC4G_HM(TA, TO)                                                                                                      \
-  heads_mfma_kernel<TA, TO, kNB><<<mgrid, kWave, 0, s>>>(static_cast<const TA*>(a), a_row, a_head, wp, static_cast<TO*>(out), \
-                                                         o_row, o_head, m, n, k)
+#define BC4G_HM(TA, TO)                                                                                                        \
+  do {                                                                                                                         \
+    if (nb == 1)                                                                                                               \
+      heads_mfma_kernel<TA, TO, 1><<<mgrid, kWave, 0, s>>>(static_cast<const TA*>(a), a_row, a_head, wp, static_cast<TO*>(out), \
+                                                           o_row, o_head, m, n, k);                                            \
+    else                                                                                                                       \
+      heads_mfma_kernel<TA, TO, 4><<<mgrid, kWave, 0, s>>>(static_cast<const TA*>(a), a_row, a_head, wp, static_cast<TO*>(out), \
+                                                           o_row, o_head, m, n, k);                                            \
+  } while (0)
     if (a_dtype == kBF16 && out_dtype == kF32) BC4G_HM(bf16_t, float);
     else if (a_dtype == kBF16) BC4G_HM(bf16_t, bf16_t);
     else if (out_dtype == kF32) BC4G_HM(float, float);

@@ -199,27 +199,39 @@ __global__ __launch_bounds__(256, 2) void latent_mfma_kernel(
   }
 }
 
-// out[row] = sum_z part_o[z][row] 2^(m_z - M) / (sum_z l_z 2^(m_z - M) + 2^(sink log2(e) - M)): one wave a (row, head).
-__global__ __launch_bounds__(kWave) void latent_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                                             const float* __restrict__ sink, float* __restrict__ out,
-                                                             long rows, int heads, int rank, int n_splits) {
+// out[row] = sum_z part_o[z][row] 2^(m_z - M) / (sum_z l_z 2^(m_z - M) + 2^(sink log2(e) - M)): a workgroup a (row, head).
+// Its first wave weighs the parts (a lane a part: at most 64), then a thread takes four numbers of the latent and asks
+// for eight parts of them at a time.
+constexpr int kMergeBlock = 128;
+__global__ __launch_bounds__(kMergeBlock) void latent_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                                   const float* __restrict__ sink, float* __restrict__ out,
+                                                                   long rows, int heads, int rank, int n_splits) {
+  __shared__ float weight[kWave + 1];
   const long row = blockIdx.x;
-  const int lane = threadIdx.x;
-  // a lane a part for the maxima and sums (at most 64 parts), then a lane a number of the latent
-  float mz = -INFINITY, lz = 0.f;
-  if (lane < n_splits) {
-    const float2 ml = *reinterpret_cast<const float2*>(part_ml + (lane * rows + row) * 2);
-    mz = ml.x, lz = ml.y;
+  if (threadIdx.x < kWave) {
+    const int lane = threadIdx.x;
+    float mz = -INFINITY, lz = 0.f;
+    if (lane < n_splits) {
+      const float2 ml = *reinterpret_cast<const float2*>(part_ml + (lane * rows + row) * 2);
+      mz = ml.x, lz = ml.y;
+    }
+    const float big = wave_max(mz);
+    const float wz = __builtin_amdgcn_exp2f(mz - big);
+    const float total = wave_sum(lz * wz) + (sink ? __builtin_amdgcn_exp2f(sink[row % heads] * kLog2e - big) : 0.f);
+    weight[lane] = wz;
+    if (lane == 0) weight[kWave] = 1.0f / total;
   }
-  const float big = wave_max(mz);
-  const float wz = __builtin_amdgcn_exp2f(mz - big);
-  const float total = wave_sum(lz * wz) + (sink ? __builtin_amdgcn_exp2f(sink[row % heads] * kLog2e - big) : 0.f);
-  const float inv = 1.0f / total;
-  for (int d = lane; d < rank; d += kWave) {
-    float sum = 0.f;
-#pragma unroll 4
-    for (int z = 0; z < n_splits; ++z) sum = fmaf(part_o[(z * rows + row) * rank + d], __shfl(wz, z, kWave), sum);
-    out[row * rank + d] = sum * inv;
+  __syncthreads();
+  const float inv = weight[kWave];
+  for (int d = 4 * threadIdx.x; d < rank; d += 4 * kMergeBlock) {
+    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 8
+    for (int z = 0; z < n_splits; ++z) {
+      const float4 v = *reinterpret_cast<const float4*>(part_o + (z * rows + row) * rank + d);
+      const float wz = weight[z];
+      sum.x = fmaf(v.x, wz, sum.x), sum.y = fmaf(v.y, wz, sum.y), sum.z = fmaf(v.z, wz, sum.z), sum.w = fmaf(v.w, wz, sum.w);
+    }
+    *reinterpret_cast<float4*>(out + row * rank + d) = make_float4(sum.x * inv, sum.y * inv, sum.z * inv, sum.w * inv);
   }
 }
 
@@ -275,7 +287,7 @@ extern "C" int bc4g_attention_latent_mfma(const float* q_lat, float* out, float*
   else { BC4G_LATENT(18, 32); }
 #undef BC4G_LATENT
   if (n_splits > 1)
-    latent_merge_kernel<<<static_cast<unsigned>(static_cast<long>(n_tokens) * heads), kWave, 0, s>>>(
+    latent_merge_kernel<<<static_cast<unsigned>(static_cast<long>(n_tokens) * heads), kMergeBlock, 0, s>>>(
         part_o, part_ml, sink, out, static_cast<long>(n_tokens) * heads, heads, rank, n_splits);
   return check_launch("attention_latent_mfma");
 }

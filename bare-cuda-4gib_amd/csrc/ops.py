@@ -1244,7 +1244,7 @@ def rglru(u: torch.Tensor, y: torch.Tensor, w_gates: torch.Tensor, ra_b: torch.T
     return out
 
 
-LATENT_MAX_ROW = 640        # numbers of a latent cache row (latent + rotated key part) the attention kernel takes
+LATENT_MAX_ROW = 1024       # numbers of a latent cache row (latent + rotated key part) the attention kernel takes
 LATENT_MFMA = True          # (off: the plain kernel also where the matrix-core kernel takes the sizes)
 LATENT_ENOUGH_GROUPS = 256  # workgroups from which on the keys are not cut into parts
 LATENT_MAX_SPLITS = 64

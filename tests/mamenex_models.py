@@ -48,8 +48,12 @@ CONFIGS: Dict[str, dict] = {
         latent(4, 16, 16, 16, 48, dims=16, ff=64),
         recurrent(64, 4, 4),
         latent(20, 8, 16, 8, 112, dims=8, base=1000.0)]),
+    "T": dict(architecture="Mamenex", vocab=64, width=32, norm=dict(eps=1e-5), canon=dict(taps=2), layers=[
+        recurrent(32, 2, 3), recurrent(48, 3, 2, ff=40)]),                         # no attention: nothing is kept per token
+    "U": dict(architecture="Mamenex", vocab=64, width=32, norm=dict(eps=1e-5), canon=dict(taps=5), layers=[
+        latent(2, 8, 8, 8, 24, dims=8), latent(6, 4, 2, 4, 10, dims=2, ff=48)]),    # no recurrence
 }
-SEEDS = {"P": 11, "Q": 22, "R": 33, "S": 44}
+SEEDS = {"P": 11, "Q": 22, "R": 33, "S": 44, "T": 55, "U": 66}
 
 
 def tensors_for(config: dict, seed: int, query_factor: float = 3.0, sink_mean: float = 0.0) -> Dict[str, torch.Tensor]:

@@ -21,7 +21,7 @@ pytestmark = pytest.mark.gpu
 # against float64 through up to four layers with peaked attention.  bfloat16: activations between kernels carry 8 bits; peaked attention multiplies what the layers before have
 # left (two keys that score alike change places), so the bfloat16 folders are drawn with smaller query weights.
 ROW_RMS = {"float32": 2e-5, "bfloat16": 5e-2}
-LENGTHS = {"P": [1, 2, 9, 70, 150], "Q": [3, 33, 64, 129], "R": [1, 17, 140], "S": [1, 5, 40, 131]}
+LENGTHS = {"P": [1, 2, 9, 70, 150], "Q": [3, 33, 64, 129], "R": [1, 17, 140], "S": [1, 5, 40, 131], "T": [1, 3, 90], "U": [2, 70]}
 
 
 def close_rows(got, where, plain_logits, dtype, label, factor=1.0):
@@ -190,6 +190,25 @@ def test_greedy_generation_through_the_entry_point_and_the_scheduler(setups, dty
             assert float(row.max() - row[tok]) <= margin, f"token {i} ({tok}) lies {row.max() - row[tok]:.4g} below the plain best"
     stats = engine.stats()
     assert stats["kv_pages_used"] == 0 and stats["running"] == 0
+
+
+def test_the_command_line_generates_from_a_folder(setups):
+    """bin/llm-infer over a Mamenex folder: the architecture is chosen by config.json, ids in, ids out."""
+    import os
+    import subprocess
+    import sys
+    folder, _, _ = setups("S", "float32")
+    config, weights = plain.load_folder(folder)
+    prompt = helpers.random_ids(9, config["vocab"], 4)
+    proc = subprocess.run([sys.executable, os.path.join(helpers.ROOT, "bin", "llm-infer"), "--model", folder, "--prompt",
+                           ",".join(map(str, prompt)), "--tokens", "6", "--dtype", "float32"], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    tokens = [int(t) for t in proc.stdout.strip().splitlines()[-1].split(":", 1)[1].split()]
+    assert len(tokens) == 6
+    full = plain.forward(config, weights, prompt + tokens).numpy()
+    for i, tok in enumerate(tokens):
+        row = full[len(prompt) - 1 + i]
+        assert float(row.max() - row[tok]) <= 1e-4, (i, tok)
 
 
 def test_the_replay_program_on_a_mixed_trace(setups, tmp_path):
