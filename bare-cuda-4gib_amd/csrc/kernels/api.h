@@ -251,10 +251,12 @@ int bc4g_rglru_scan(const float* pre, const void* u, const void* y, int dtype, c
 // cache slot (slot_map[t] = page * page_tokens + offset; cache [pages, page_tokens, rank + rot]; null: nothing is
 // written) receives [rmsnorm(dkv[:rank]) * g | rotate(dkv[rank:])], and q_lat [T, heads, rank + rot] (float32) the
 // rotated part of every head's query in its last rot numbers.  Elements 2i and 2i + 1 of the first `dims` numbers of
-// a rotated part turn by position * base^(-2i / dims).
-int bc4g_latent_prepare(const void* q, const void* dkv, int dtype, const float* g, float eps, const int32_t* positions,
+// a rotated part turn by position * base^(-2i / dims): angles [T, dims / 2, 2] holds every row's cosines and sines
+// (bc4g_latent_angles makes it, the angles worked out in double: once a step for all layers of one rotation).
+int bc4g_latent_angles(const int32_t* positions, float* table, int n_rows, int dims, float base, void* stream);
+int bc4g_latent_prepare(const void* q, const void* dkv, int dtype, const float* g, float eps, const float* angles,
                         const int32_t* slot_map, void* cache, float* q_lat, int n_rows, int heads, int plain, int rot,
-                        int rank, int dims, float base, void* stream);
+                        int rank, int dims, void* stream);
 // out[t, h, :n] = w[h] a[t, h, :k] for every head: a at a + t * a_row + h * a_head, out likewise, w [heads, n, k].
 int bc4g_heads_gemm(const void* a, int a_dtype, long a_row, long a_head, const void* w, int w_dtype, void* out, int out_dtype,
                     long o_row, long o_head, int m, int n, int k, int heads, void* stream);

@@ -32,19 +32,30 @@ __device__ inline void pair_angle(int pos, int i, int dims, double log_base, flo
   *s = static_cast<float>(sd);
 }
 
+// The step's table of angles, for every layer with the same rotation to share: table[t][i] = (cos, sin) of pair i at
+// the row's position.
+__global__ void latent_angles_kernel(const int32_t* __restrict__ positions, float2* __restrict__ table, long total, int half,
+                                     double log_base) {
+  const long stride = static_cast<long>(blockDim.x) * gridDim.x;
+  for (long idx = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; idx < total; idx += stride) {
+    float c, s;
+    pair_angle(positions[idx / half], static_cast<int>(idx % half), 2 * half, log_base, &c, &s);
+    table[idx] = make_float2(c, s);
+  }
+}
+
 // One workgroup a row.  q: [T, heads, plain + rot] (as projected); dkv: [T, rank + rot]; q_lat: [T, heads, rank + rot]
 // float, of which this kernel writes the last rot of every head; the row's cache slot receives [normed latent | rotated
 // key part].  Neighbouring elements 2i and 2i + 1 of the first `dims` of a rotated part are a pair; the rest passes.
 template <typename T>
 __global__ __launch_bounds__(kPrepBlock) void latent_prepare_kernel(
     const T* __restrict__ q, const T* __restrict__ dkv, const float* __restrict__ g, float eps,
-    const int32_t* __restrict__ positions, const int32_t* __restrict__ slot_map, T* __restrict__ cache,
-    float* __restrict__ q_lat, int heads, int plain, int rot, int rank, int dims, double log_base) {
+    const float* __restrict__ angles, const int32_t* __restrict__ slot_map, T* __restrict__ cache,
+    float* __restrict__ q_lat, int heads, int plain, int rot, int rank, int dims) {
   __shared__ float scratch[16];
   extern __shared__ float cs[];                     // [dims / 2][2]: the row's cosines and sines
   const long row = blockIdx.x;
-  const int pos = positions[row];
-  for (int i = threadIdx.x; i < dims / 2; i += kPrepBlock) pair_angle(pos, i, dims, log_base, &cs[2 * i], &cs[2 * i + 1]);
+  for (int i = threadIdx.x; i < dims; i += kPrepBlock) cs[i] = angles[row * dims + i];
   const T* lat = dkv + row * (rank + rot);
   float ss = 0.f;
   for (int i = threadIdx.x; i < rank; i += kPrepBlock) {
@@ -134,12 +145,16 @@ __device__ inline uint4 load_slots(const float* p) {
   return make_uint4(two(a.x, a.y), two(a.z, a.w), two(b.x, b.y), two(b.z, b.w));
 }
 
-template <typename TA, typename TO, int NB>
-__global__ __launch_bounds__(kWave) void heads_mfma_kernel(const TA* __restrict__ a, long a_row, long a_head,
-                                                           const bf16_t* __restrict__ w, TO* __restrict__ out, long o_row,
-                                                           long o_head, int m, int n, int k) {
+// KW waves of a workgroup take every KW-th k-step and add their sums up through LDS (few rows: more waves on the
+// weights' way in).
+template <typename TA, typename TO, int NB, int KW>
+__global__ __launch_bounds__(kWave * KW) void heads_mfma_kernel(const TA* __restrict__ a, long a_row, long a_head,
+                                                                const bf16_t* __restrict__ w, TO* __restrict__ out, long o_row,
+                                                                long o_head, int m, int n, int k) {
+  __shared__ floatx4 sums[KW > 1 ? KW : 1][NB][kWave];
   const int h = blockIdx.z, m0 = blockIdx.x * 16, n0 = blockIdx.y * 16 * NB;
-  const int c = threadIdx.x % 16, g = threadIdx.x / 16;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int c = lane % 16, g = lane / 16;
   const bool row_there = m0 + c < m;
   const TA* arow = a + (m0 + c) * a_row + h * a_head + 8 * g;
   const bf16_t* wcol[NB];
@@ -153,7 +168,7 @@ __global__ __launch_bounds__(kWave) void heads_mfma_kernel(const TA* __restrict_
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) acc[nb] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll 8
-  for (int k0 = 0; k0 < k; k0 += 32) {
+  for (int k0 = 32 * wave; k0 < k; k0 += 32 * KW) {
     const bool k_there = k0 + 8 * g < k;
     const uint4 av = row_there && k_there ? load_slots(arow + k0) : zero16();
 #pragma unroll
@@ -161,6 +176,16 @@ __global__ __launch_bounds__(kWave) void heads_mfma_kernel(const TA* __restrict_
       const uint4 wv = col_there[nb] && k_there ? load16(wcol[nb] + k0) : zero16();
       acc[nb] = mfma_16x16x32(av, wv, acc[nb]);
     }
+  }
+  if (KW > 1) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) sums[wave][nb][lane] = acc[nb];
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int other = 1; other < KW; ++other) acc[nb] += sums[other][nb][lane];
   }
   // a lane holds column c of every block and rows 4g .. 4g + 3
 #pragma unroll
@@ -275,26 +300,36 @@ __global__ void attention_latent_kernel(const float* __restrict__ q_lat, float* 
 
 using namespace bc4g;
 
+extern "C" int bc4g_latent_angles(const int32_t* positions, float* table, int n_rows, int dims, float base, void* stream) {
+  BC4G_REQUIRE(n_rows >= 0 && dims > 0 && dims % 2 == 0 && base > 0.f && positions && table,
+               "latent_angles: bad arguments (T=%d, %d rotated dimensions, base %g)", n_rows, dims, base);
+  if (n_rows == 0) return 0;
+  const long total = static_cast<long>(n_rows) * (dims / 2);
+  const long blocks = (total + 255) / 256;
+  latent_angles_kernel<<<static_cast<unsigned>(blocks > 65535 ? 65535 : blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(
+      positions, reinterpret_cast<float2*>(table), total, dims / 2, log(static_cast<double>(base)));
+  return check_launch("latent_angles");
+}
+
 extern "C" int bc4g_latent_prepare(const void* q, const void* dkv, int dtype, const float* g, float eps,
-                                   const int32_t* positions, const int32_t* slot_map, void* cache, float* q_lat,
-                                   int n_rows, int heads, int plain, int rot, int rank, int dims, float base, void* stream) {
+                                   const float* angles, const int32_t* slot_map, void* cache, float* q_lat,
+                                   int n_rows, int heads, int plain, int rot, int rank, int dims, void* stream) {
   BC4G_REQUIRE(n_rows >= 0 && heads > 0 && plain >= 0 && rot >= 0 && rank > 0, "latent_prepare: bad sizes T=%d heads=%d "
                "plain=%d rot=%d rank=%d", n_rows, heads, plain, rot, rank);
-  BC4G_REQUIRE(dims >= 0 && dims % 2 == 0 && dims <= rot && dims <= 8192 && base > 0.f,
-               "latent_prepare: %d rotated dimensions of %d (even, at most the rotated part) with base %g", dims, rot, base);
-  BC4G_REQUIRE(q && dkv && g && positions && q_lat && (!cache || slot_map), "latent_prepare: a tensor is missing");
+  BC4G_REQUIRE(dims >= 0 && dims % 2 == 0 && dims <= rot && dims <= 8192,
+               "latent_prepare: %d rotated dimensions of %d (even, at most the rotated part)", dims, rot);
+  BC4G_REQUIRE(q && dkv && g && (angles || dims == 0) && q_lat && (!cache || slot_map), "latent_prepare: a tensor is missing");
   if (n_rows == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const size_t lds = static_cast<size_t>(dims > 0 ? dims : 2) * sizeof(float);
-  const double log_base = log(static_cast<double>(base));
   if (dtype == kF32)
     latent_prepare_kernel<float><<<n_rows, kPrepBlock, lds, s>>>(static_cast<const float*>(q), static_cast<const float*>(dkv), g,
-                                                                 eps, positions, slot_map, static_cast<float*>(cache), q_lat,
-                                                                 heads, plain, rot, rank, dims, log_base);
+                                                                 eps, angles, slot_map, static_cast<float*>(cache), q_lat,
+                                                                 heads, plain, rot, rank, dims);
   else if (dtype == kBF16)
     latent_prepare_kernel<bf16_t><<<n_rows, kPrepBlock, lds, s>>>(static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(dkv),
-                                                                  g, eps, positions, slot_map, static_cast<bf16_t*>(cache),
-                                                                  q_lat, heads, plain, rot, rank, dims, log_base);
+                                                                  g, eps, angles, slot_map, static_cast<bf16_t*>(cache),
+                                                                  q_lat, heads, plain, rot, rank, dims);
   else return fail("latent_prepare: unknown dtype %d", dtype);
   return check_launch("latent_prepare");
 }
@@ -318,11 +353,11 @@ extern "C" int bc4g_heads_gemm(const void* a, int a_dtype, long a_row, long a_he
 #define BC4G_HM(TA, TO)                                                                                                        \
   do {                                                                                                                         \
     if (nb == 1)                                                                                                               \
-      heads_mfma_kernel<TA, TO, 1><<<mgrid, kWave, 0, s>>>(static_cast<const TA*>(a), a_row, a_head, wp, static_cast<TO*>(out), \
-                                                           o_row, o_head, m, n, k);                                            \
+      heads_mfma_kernel<TA, TO, 1, 4><<<mgrid, 4 * kWave, 0, s>>>(static_cast<const TA*>(a), a_row, a_head, wp,                \
+                                                                  static_cast<TO*>(out), o_row, o_head, m, n, k);              \
     else                                                                                                                       \
-      heads_mfma_kernel<TA, TO, 4><<<mgrid, kWave, 0, s>>>(static_cast<const TA*>(a), a_row, a_head, wp, static_cast<TO*>(out), \
-                                                           o_row, o_head, m, n, k);                                            \
+      heads_mfma_kernel<TA, TO, 4, 1><<<mgrid, kWave, 0, s>>>(static_cast<const TA*>(a), a_row, a_head, wp,                    \
+                                                              static_cast<TO*>(out), o_row, o_head, m, n, k);                  \
   } while (0)
     if (a_dtype == kBF16 && out_dtype == kF32) BC4G_HM(bf16_t, float);
     else if (a_dtype == kBF16) BC4G_HM(bf16_t, bf16_t);

@@ -199,6 +199,169 @@ __global__ __launch_bounds__(256, 2) void latent_mfma_kernel(
   }
 }
 
+// The form for few rows (a decode step): a workgroup takes ONE tile of 16 (token, head) pairs and its four waves cut
+// the tile's work between them -- wave w the k-steps w, w + 4, ... of the scores (the partial scores are added up
+// through LDS, every wave in the same order, so all four hold the same bits and take the same maximum and sum) and
+// the blocks w, w + 4, ... of the latent for the output.  A wave then keeps a quarter of the queries and of the sums
+// in registers, and a tile's chain of LDS reads and matrix instructions is a quarter as long.
+template <int KS, int DB>
+__global__ __launch_bounds__(256) void latent_mfma_shared_kernel(
+    const float* __restrict__ q_lat, float* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const bf16_t* __restrict__ cache, const float* __restrict__ sink, const int32_t* __restrict__ block_table,
+    int table_stride, const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_ctx, int n_tokens, int heads,
+    int rank, int dk, int page_tokens, int window, float scale, int hb, int tpt, int n_hg, int n_splits) {
+  extern __shared__ uint4 tile[];                             // the tile, its latent part transposed, the partial scores
+  constexpr int KW = (KS + 3) / 4, DW = (DB + 3) / 4;         // k-steps and latent blocks of a wave
+  const int s = blockIdx.y, z = blockIdx.z;
+  const int tok0 = seq_start[s], n_tok = seq_start[s + 1] - tok0, cached = seq_ctx[s];
+  const int n_tb = (n_tok + tpt - 1) / tpt, n_tiles = n_tb * n_hg;
+  const int my_tile = blockIdx.x;
+  if (my_tile >= n_tiles) return;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int tb = my_tile / n_hg, hg = my_tile % n_hg;
+  const int c = lane % 16, g = lane / 16;
+  const int tq = tb * tpt + c / hb, head = hg * hb + c % hb;
+  const bool q_live = c / hb < tpt && tq < n_tok && head < heads;
+  const int pos = cached + tq;
+  const int32_t* table = block_table + static_cast<long>(s) * table_stride;
+  const int cpr = dk / 8, pitch = cpr + 1;
+  const int last_pos = cached + min(n_tok, (tb + 1) * tpt) - 1;
+  const int first_pos = window > 0 ? max(0, cached + tb * tpt - window + 1) : 0;
+  const int kt_begin = first_pos / kKeys, kt_end = last_pos / kKeys + 1;
+  const int per = (kt_end - kt_begin + n_splits - 1) / n_splits;
+  const int kt_lo = kt_begin + z * per, kt_hi = min(kt_end, kt_lo + per);
+
+  uint4 qf[KW];
+  {
+    const float* qrow = q_lat + (static_cast<long>(tok0 + tq) * heads + head) * dk;
+#pragma unroll
+    for (int i = 0; i < KW; ++i) {
+      const int ks = wave + 4 * i;
+      qf[i] = zero16();
+      if (q_live && ks * 32 < dk) {
+        const float4 a = *reinterpret_cast<const float4*>(qrow + ks * 32 + 8 * g);
+        const float4 b = *reinterpret_cast<const float4*>(qrow + ks * 32 + 8 * g + 4);
+        qf[i] = make_uint4(pack_bf16(a.x, a.y), pack_bf16(a.z, a.w), pack_bf16(b.x, b.y), pack_bf16(b.z, b.w));
+      }
+    }
+  }
+  floatx4 acc[DW];
+#pragma unroll
+  for (int i = 0; i < DW; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const float scale2 = scale * kLog2e;
+  uint16_t* vt = reinterpret_cast<uint16_t*>(tile + kKeys * pitch);
+  float4* partial = reinterpret_cast<float4*>(reinterpret_cast<char*>(tile) + kKeys * pitch * 16 + ((rank * kVtPitch * 2 + 15) / 16) * 16);
+
+  constexpr int kPieces = (KS * 4 + 7) / 8;
+  const int st_key = threadIdx.x / 8, st_sub = threadIdx.x % 8;
+  uint4 stage[kPieces];
+  for (int kt = kt_lo; kt < kt_hi; ++kt) {
+    const int j0 = kt * kKeys;
+    {
+      const int j = j0 + st_key;
+      const bool there = j >= first_pos && j <= last_pos;
+      const bf16_t* src = cache;
+      if (there) src = cache + (static_cast<long>(table[j / page_tokens]) * page_tokens + j % page_tokens) * dk;
+#pragma unroll
+      for (int p = 0; p < kPieces; ++p) {
+        const int part = st_sub + 8 * p;
+        stage[p] = there && part < cpr ? load16(src + part * 8) : zero16();
+      }
+    }
+#pragma unroll
+    for (int p = 0; p < kPieces; ++p) {
+      const int part = st_sub + 8 * p;
+      if (part < cpr) tile[st_key * pitch + part] = stage[p];
+      if (part * 8 < rank) {
+        uint16_t* to = vt + part * 8 * kVtPitch + st_key;
+        const unsigned w[4] = {stage[p].x, stage[p].y, stage[p].z, stage[p].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          to[(2 * e) * kVtPitch] = static_cast<uint16_t>(w[e] & 0xffffu);
+          to[(2 * e + 1) * kVtPitch] = static_cast<uint16_t>(w[e] >> 16);
+        }
+      }
+    }
+    lds_barrier();
+    floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < KW; ++i) {
+      const int ks = wave + 4 * i;
+      if (ks * 32 < dk) {
+        s0 = mfma_16x16x32(tile[c * pitch + ks * 4 + g], qf[i], s0);
+        s1 = mfma_16x16x32(tile[(16 + c) * pitch + ks * 4 + g], qf[i], s1);
+      }
+    }
+    partial[(wave * kWave + lane) * 2] = make_float4(s0[0], s0[1], s0[2], s0[3]);
+    partial[(wave * kWave + lane) * 2 + 1] = make_float4(s1[0], s1[1], s1[2], s1[3]);
+    lds_barrier();
+    float p[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) p[i] = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {                             // (in this order in every wave)
+      const float4 a = partial[(w * kWave + lane) * 2], b = partial[(w * kWave + lane) * 2 + 1];
+      p[0] += a.x, p[1] += a.y, p[2] += a.z, p[3] += a.w, p[4] += b.x, p[5] += b.y, p[6] += b.z, p[7] += b.w;
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int j = j0 + (i < 4 ? 0 : 16) + 4 * g + (i & 3);
+      const bool seen = q_live && j <= pos && (window == 0 || j > pos - window);
+      p[i] = seen ? p[i] * scale2 : -INFINITY;
+      mx = fmaxf(mx, p[i]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    const float m_new = fmaxf(m, mx);
+    const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      p[i] = p[i] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(p[i] - m_new);
+      sum += p[i];
+    }
+    l = l * alpha + sum;
+    m = m_new;
+#pragma unroll
+    for (int i = 0; i < DW; ++i) acc[i] *= alpha;
+    const uint4 pf = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
+    const uint16_t* col = vt + c * kVtPitch + 4 * g;
+#pragma unroll
+    for (int i = 0; i < DW; ++i) {
+      const int db = wave + 4 * i;
+      if (db * 16 < rank) {
+        const uint2 lo = *reinterpret_cast<const uint2*>(col + db * 16 * kVtPitch);
+        const uint2 hi = *reinterpret_cast<const uint2*>(col + db * 16 * kVtPitch + 16);
+        acc[i] = mfma_16x16x32(make_uint4(lo.x, lo.y, hi.x, hi.y), pf, acc[i]);
+      }
+    }
+    lds_barrier();                                            // the tile has been read by everyone
+  }
+  if (!q_live) return;
+  l += __shfl_xor(l, 16, kWave);
+  l += __shfl_xor(l, 32, kWave);
+  const long row = static_cast<long>(tok0 + tq) * heads + head;
+  float inv = 1.f;
+  float* o = part_o + (static_cast<long>(z) * n_tokens * heads + row) * rank;
+  if (n_splits == 1) {
+    if (sink) l += __builtin_amdgcn_exp2f(sink[head] * kLog2e - m);
+    inv = 1.0f / l;
+    o = out + row * rank;
+  } else if (wave == 0 && g == 0) {
+    float* ml = part_ml + (static_cast<long>(z) * n_tokens * heads + row) * 2;
+    ml[0] = m;
+    ml[1] = l;
+  }
+#pragma unroll
+  for (int i = 0; i < DW; ++i) {
+    const int db = wave + 4 * i;
+    if (db * 16 < rank)
+      *reinterpret_cast<float4*>(o + db * 16 + 4 * g) = make_float4(acc[i][0] * inv, acc[i][1] * inv, acc[i][2] * inv, acc[i][3] * inv);
+  }
+}
+
 // out[row] = sum_z part_o[z][row] 2^(m_z - M) / (sum_z l_z 2^(m_z - M) + 2^(sink log2(e) - M)): a workgroup a (row, head).
 // Its first wave weighs the parts (a lane a part: at most 64), then a thread takes four numbers of the latent and asks
 // for eight parts of them at a time.
@@ -270,18 +433,30 @@ extern "C" int bc4g_attention_latent_mfma(const float* q_lat, float* out, float*
   const int hb = heads < 16 ? heads : 16, tpt = 16 / hb, n_hg = ceil_div(heads, hb);
   const int most_tiles = ceil_div(most_tokens, tpt) * n_hg;
   BC4G_REQUIRE(n_seqs <= 65535 && n_splits <= 65535, "attention_latent_mfma: %d requests are beyond the grid limit", n_seqs);
-  dim3 grid(ceil_div(most_tiles, 4), n_seqs, n_splits);
-  const size_t lds = static_cast<size_t>(kKeys) * (dk / 8 + 1) * 16 + static_cast<size_t>(rank) * kVtPitch * 2;
+  // no request with four tiles (a decode step): a workgroup a tile, the waves cut the tile's work
+  const bool shared = most_tiles < 4;
+  dim3 grid(shared ? most_tiles : ceil_div(most_tiles, 4), n_seqs, n_splits);
+  const size_t lds = static_cast<size_t>(kKeys) * (dk / 8 + 1) * 16 + (static_cast<size_t>(rank) * kVtPitch * 2 + 15) / 16 * 16 +
+                     (shared ? 4 * kWave * 32 : 0);
   const bf16_t* kc = static_cast<const bf16_t*>(cache);
   // (more than 64 KB of LDS a workgroup has to be asked for, once for a kernel: the most this kernel ever takes)
 #define BC4G_LATENT(KS, DB)                                                                                                 \
   static const hipError_t allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_mfma_kernel<KS, DB>),         \
                                                         hipFuncAttributeMaxDynamicSharedMemorySize,                          \
                                                         kKeys * (KS * 4 + 1) * 16 + DB * 16 * kVtPitch * 2);                 \
-  BC4G_REQUIRE(allowed == hipSuccess, "attention_latent_mfma: %zu bytes of LDS a workgroup are refused", lds);              \
-  latent_mfma_kernel<KS, DB><<<grid, 256, lds, s>>>(q_lat, out, part_o, part_ml, kc, sink, block_table, table_stride, seq_start, \
-                                                    seq_ctx, n_tokens, heads, rank, dk, page_tokens, window, scale, hb, tpt, n_hg, \
-                                                    n_splits)
+  static const hipError_t allowed_shared = hipFuncSetAttribute(                                                              \
+      reinterpret_cast<const void*>(&latent_mfma_shared_kernel<KS, DB>), hipFuncAttributeMaxDynamicSharedMemorySize,         \
+      kKeys * (KS * 4 + 1) * 16 + DB * 16 * kVtPitch * 2 + 4 * kWave * 32);                                                  \
+  BC4G_REQUIRE(allowed == hipSuccess && allowed_shared == hipSuccess,                                                        \
+               "attention_latent_mfma: %zu bytes of LDS a workgroup are refused", lds);                                       \
+  if (shared)                                                                                                                 \
+    latent_mfma_shared_kernel<KS, DB><<<grid, 256, lds, s>>>(q_lat, out, part_o, part_ml, kc, sink, block_table, table_stride, \
+                                                             seq_start, seq_ctx, n_tokens, heads, rank, dk, page_tokens, window, \
+                                                             scale, hb, tpt, n_hg, n_splits);                                 \
+  else                                                                                                                        \
+    latent_mfma_kernel<KS, DB><<<grid, 256, lds, s>>>(q_lat, out, part_o, part_ml, kc, sink, block_table, table_stride, seq_start, \
+                                                      seq_ctx, n_tokens, heads, rank, dk, page_tokens, window, scale, hb, tpt, n_hg, \
+                                                      n_splits)
   if (dk <= 128 && rank <= 64) { BC4G_LATENT(4, 4); }
   else if (dk <= 320 && rank <= 256) { BC4G_LATENT(10, 16); }
   else { BC4G_LATENT(18, 32); }

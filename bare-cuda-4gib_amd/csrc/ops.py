@@ -1264,32 +1264,48 @@ def latent_splits(seq_start, heads: int, max_kv_len: int) -> int:
     the workgroups to twice that, while a part keeps a key tile of 32."""
     hb = min(heads, 16)
     tpt, n_hg = 16 // hb, -(-heads // hb)
-    groups = sum(-(-(-(-int(seq_start[s + 1] - seq_start[s]) // tpt) * n_hg) // 4) for s in range(len(seq_start) - 1))
+    tiles = [-(-int(seq_start[s + 1] - seq_start[s]) // tpt) * n_hg for s in range(len(seq_start) - 1)]
+    # (no request with four tiles: a workgroup a tile, else four tiles a workgroup)
+    groups = sum(tiles) if max(tiles, default=0) < 4 else sum(-(-n // 4) for n in tiles)
     if groups >= LATENT_ENOUGH_GROUPS or groups == 0:
         return 1
     key_tiles = -(-max_kv_len // 32)
     return max(1, min(-(-2 * LATENT_ENOUGH_GROUPS // groups), key_tiles, LATENT_MAX_SPLITS))
 
 
-def latent_prepare(q: torch.Tensor, dkv: torch.Tensor, g: torch.Tensor, eps: float, positions: torch.Tensor,
+def latent_angles(positions: torch.Tensor, dims: int, base: float) -> torch.Tensor:
+    """(cos, sin) of every row's angles position * base^(-2i / dims), float32 [T, dims / 2, 2], worked out in double:
+    made once a step and read by every layer that rotates alike."""
+    _dev("latent_angles", positions)
+    t = positions.shape[0]
+    _i32("latent_angles", "positions", positions, t)
+    table = torch.empty((t, dims // 2, 2), dtype=torch.float32, device=positions.device)
+    library.call("bc4g_latent_angles", _ptr(positions), _ptr(table), t, int(dims), float(base), _stream(),
+                 cost=lambda: (0.0, t * dims * 4))
+    return table
+
+
+def latent_prepare(q: torch.Tensor, dkv: torch.Tensor, g: torch.Tensor, eps: float, angles: Optional[torch.Tensor],
                    slot_map: Optional[torch.Tensor], cache: Optional[torch.Tensor], q_lat: torch.Tensor, heads: int, plain: int,
-                   rot: int, rank: int, dims: int, base: float) -> None:
+                   rot: int, rank: int, dims: int) -> None:
     """Writes [rmsnorm(dkv[:, :rank]) * g | rotate(dkv[:, rank:])] into every row's cache slot (``cache`` None: nowhere)
-    and every head's rotated query part into q_lat[:, h, rank:]."""
-    _dev("latent_prepare", q, dkv, g, positions, slot_map, cache, q_lat)
+    and every head's rotated query part into q_lat[:, h, rank:].  ``angles``: latent_angles of the rows (None where
+    nothing is rotated, dims 0)."""
+    _dev("latent_prepare", q, dkv, g, angles, slot_map, cache, q_lat)
     t = q.shape[0]
     if q.dtype != dkv.dtype or tuple(q.shape) != (t, heads * (plain + rot)) or tuple(dkv.shape) != (t, rank + rot):
         raise KernelError(f"latent_prepare: q {tuple(q.shape)} / dkv {tuple(dkv.shape)} do not fit heads={heads} plain={plain} rot={rot} rank={rank}")
     _f32("latent_prepare", "g", g, (rank,))
     _f32("latent_prepare", "q_lat", q_lat, (t, heads, rank + rot))
-    _i32("latent_prepare", "positions", positions, t)
+    if dims:
+        _f32("latent_prepare", "angles", angles, (t, dims // 2, 2))
     if cache is not None:
         if cache.dtype != q.dtype or cache.dim() != 3 or cache.shape[2] != rank + rot:
             raise KernelError(f"latent_prepare: the cache must be {q.dtype} [pages, page_tokens, {rank + rot}], got {cache.dtype} {tuple(cache.shape)}")
         _i32("latent_prepare", "slot_map", slot_map, t)
-    library.call("bc4g_latent_prepare", _ptr(q), _ptr(dkv), _code(q, "latent_prepare"), _ptr(g), float(eps), _ptr(positions),
-                 _ptr(slot_map) if cache is not None else None, _ptr(cache), _ptr(q_lat), t, heads, plain, rot, rank, int(dims),
-                 float(base), _stream(), cost=lambda: (4.0 * t * (rank + (heads + 1) * rot), t * (q.element_size() * (heads + 2) * rot + 2 * rank * q.element_size())))
+    library.call("bc4g_latent_prepare", _ptr(q), _ptr(dkv), _code(q, "latent_prepare"), _ptr(g), float(eps),
+                 _ptr(angles) if dims else None, _ptr(slot_map) if cache is not None else None, _ptr(cache), _ptr(q_lat), t, heads,
+                 plain, rot, rank, int(dims), _stream(), cost=lambda: (4.0 * t * (rank + (heads + 1) * rot), t * (q.element_size() * (heads + 2) * rot + 2 * rank * q.element_size())))
 
 
 def heads_gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, k: int, n: int) -> None:

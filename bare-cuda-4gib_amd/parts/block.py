@@ -88,7 +88,9 @@ class SandwichBlock(Part):
         self.mixer_post_norm.add_to(x, y)
         if self.ffn is not None:
             y = torch.zeros_like(x)
-            self.ffn.forward(self.ffn_norm.forward(x, ctx), ctx, y)
+            # (a feed-forward that says so gets the norm not yet computed: its first product absorbs it for few rows)
+            lazy = getattr(self.ffn, "accepts_lazy_norm", False)
+            self.ffn.forward(Normed(x, self.ffn_norm, ctx) if lazy else self.ffn_norm.forward(x, ctx), ctx, y)
             self.ffn_post_norm.add_to(x, y)
 
 

@@ -59,6 +59,7 @@ class DenseXIELU(Part):
     (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2 otherwise; p and q are the two numbers of the tensor ``act``."""
     category = "feedforward"
     graph_safe = True     # launches kernels only: may run inside a captured graph
+    accepts_lazy_norm = True
 
     def __init__(self, hidden_size: int, intermediate_size: int):
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)

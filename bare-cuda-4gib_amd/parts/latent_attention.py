@@ -81,8 +81,12 @@ class LatentAttention(Part):
         q = linear(h, self.w_q, out_dtype=self.act_dtype)
         dkv = linear(h, self.w_dkv, out_dtype=self.act_dtype)
         q_lat = torch.empty((t, H, rank + rot), dtype=torch.float32, device=q.device)
-        ops.latent_prepare(q, dkv, self.g, self.eps, ctx.positions, ctx.slot_maps[cache.group] if writes else None,
-                           cache.latent if writes else None, q_lat, H, self.dim, rot, rank, self.rot_dims, self.rot_base)
+        angles = None
+        if self.rot_dims:                 # the same in every layer that rotates alike: a table made once a step
+            angles = ctx.shared(("latent_angles", self.rot_dims, self.rot_base),
+                                lambda: ops.latent_angles(ctx.positions, self.rot_dims, self.rot_base))
+        ops.latent_prepare(q, dkv, self.g, self.eps, angles, ctx.slot_maps[cache.group] if writes else None,
+                           cache.latent if writes else None, q_lat, H, self.dim, rot, rank, self.rot_dims)
         ops.heads_gemm(q.view(t, H, self.dim + rot), self.uk_t, q_lat, k=self.dim, n=rank)
         mixed = ops.attention_latent(q_lat, cache.latent, self.sinks, ctx.block_tables[cache.group], ctx, H, rank, rot,
                                      cache.page_tokens, self.window, self.scale)

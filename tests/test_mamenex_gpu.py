@@ -369,8 +369,8 @@ def test_latent_rows_are_normed_rotated_and_written_to_their_slots(dtype):
     slot_map = torch.tensor([9, 2, 0, 7, 5], dtype=torch.int32)
     cache = torch.zeros(3, P, rank + dr, dtype=dtype, device=dev)
     q_lat = torch.zeros(T, H, rank + dr, device=dev)
-    ops.latent_prepare(q.to(dev), dkv.to(dev), g.to(dev), 1e-4, positions.to(dev), slot_map.to(dev), cache, q_lat, H, dn, dr, rank,
-                       dims, base)
+    angles = ops.latent_angles(positions.to(dev), dims, base)
+    ops.latent_prepare(q.to(dev), dkv.to(dev), g.to(dev), 1e-4, angles, slot_map.to(dev), cache, q_lat, H, dn, dr, rank, dims)
     c = plain.plain_rmsnorm(dkv[:, :rank].double(), g.double(), 1e-4)
     kr = plain.interleaved_rotation(dkv[:, rank:].double(), positions.long(), base, dims)
     qr = plain.interleaved_rotation(q.double().view(T, H, dn + dr)[..., dn:], positions.long(), base, dims)
