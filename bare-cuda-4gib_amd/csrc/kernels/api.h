@@ -229,7 +229,8 @@ int bc4g_rmsnorm_add(float* x, const void* y, int y_dtype, const float* w, int n
 int bc4g_xielu(const void* in, void* out, int dtype, const float* pq, long total, void* stream);
 
 // A causal convolution over time on each channel, across steps: out[t, c] = (add_input ? in[t, c] : 0) + out_bias[c] +
-// sum_j w[c, j] * input(t - taps + 1 + j)[c], where a row's input is in[row] + in_bias (rounded to the storage type) and
+// sum_j w[j, c] * input(t - taps + 1 + j)[c] (w comes by taps, [taps][channels], so that neighbouring channels lie side
+// by side; its last row is the current token's), where a row's input is in[row] + in_bias (rounded to the storage type) and
 // the inputs before a step's first row come from the request's state [slots, taps - 1, channels] (zero when the request
 // was admitted: zeros before the sequence).  Afterwards the state holds the request's last taps - 1 inputs.  The
 // step's rows are grouped by request: row_seq [T], seq_start [S + 1], seq_slots [S].  w, biases: float32.

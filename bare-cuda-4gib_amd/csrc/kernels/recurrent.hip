@@ -7,6 +7,7 @@
 
 #include "api.h"
 #include "common.h"
+#include "mfma.h"
 
 namespace bc4g {
 namespace {
@@ -26,7 +27,7 @@ __device__ inline float conv_input(const T* in, const float* in_bias, long at, i
   return in_bias ? to_float(from_float<T>(v + in_bias[c])) : v;
 }
 
-// out[t, c] = (add_input ? in[t, c] : 0) + out_bias[c] + sum_j w[c, j] * input(t - taps + 1 + j)[c]
+// out[t, c] = (add_input ? in[t, c] : 0) + out_bias[c] + sum_j w[j, c] * input(t - taps + 1 + j)[c]   (w: [taps][channels])
 template <typename T>
 __global__ void causal_conv_kernel(const T* __restrict__ in, const float* __restrict__ in_bias,
                                    const float* __restrict__ w, const float* __restrict__ out_bias, int add_input,
@@ -46,10 +47,67 @@ __global__ void causal_conv_kernel(const T* __restrict__ in, const float* __rest
       const int src = local - (taps - 1) + j;
       const float v = src >= 0 ? conv_input(in, in_bias, start + src, c, channels)
                                : to_float(tail[static_cast<long>(taps - 1 + src) * channels + c]);
-      acc = fmaf(w[static_cast<long>(c) * taps + j], v, acc);
+      acc = fmaf(w[static_cast<long>(j) * channels + c], v, acc);
     }
     if (add_input) acc += to_float(in[idx]);
     out[idx] = from_float<T>(acc);
+  }
+}
+
+// The same for bfloat16 and channels in whole pieces of 16 bytes: a thread takes eight channels of one row, the index
+// arithmetic once for the eight.
+__device__ inline void widen8(const uint4 v, float (&f)[8]) {
+  const unsigned w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) f[2 * e] = __uint_as_float(w[e] << 16), f[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+}
+
+__global__ void causal_conv_pieces_kernel(const bf16_t* __restrict__ in, const float* __restrict__ in_bias,
+                                          const float* __restrict__ w, const float* __restrict__ out_bias, int add_input,
+                                          bf16_t* __restrict__ out, const bf16_t* __restrict__ state,
+                                          const int32_t* __restrict__ row_seq, const int32_t* __restrict__ seq_start,
+                                          const int32_t* __restrict__ seq_slots, long total, int channels, int taps) {
+  const int pieces = channels / 8;
+  const long stride = static_cast<long>(blockDim.x) * gridDim.x;
+  for (long idx = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; idx < total; idx += stride) {
+    const int c0 = static_cast<int>(idx % pieces) * 8;
+    const long t = idx / pieces;
+    const int s = row_seq[t];
+    const long start = seq_start[s];
+    const int local = static_cast<int>(t - start);
+    const bf16_t* tail = state + static_cast<long>(seq_slots[s]) * (taps - 1) * channels;
+    float acc[8], bias[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = out_bias ? out_bias[c0 + e] : 0.f, bias[e] = in_bias ? in_bias[c0 + e] : 0.f;
+    for (int j = 0; j < taps; ++j) {
+      const int src = local - (taps - 1) + j;
+      float v[8];
+      if (src >= 0) {
+        widen8(load16(in + (start + src) * channels + c0), v);
+        if (in_bias) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] = to_float(from_float<bf16_t>(v[e] + bias[e]));      // as the tail keeps it
+        }
+      } else {
+        widen8(load16(tail + static_cast<long>(taps - 1 + src) * channels + c0), v);
+      }
+      const float4 wa = *reinterpret_cast<const float4*>(w + static_cast<long>(j) * channels + c0);
+      const float4 wb = *reinterpret_cast<const float4*>(w + static_cast<long>(j) * channels + c0 + 4);
+      const float wj[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = fmaf(wj[e], v[e], acc[e]);
+    }
+    if (add_input) {
+      float v[8];
+      widen8(load16(in + t * channels + c0), v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += v[e];
+    }
+    unsigned o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      o[e] = static_cast<unsigned>(bf16_bits_from_float(acc[2 * e])) | (static_cast<unsigned>(bf16_bits_from_float(acc[2 * e + 1])) << 16);
+    *reinterpret_cast<uint4*>(out + t * channels + c0) = make_uint4(o[0], o[1], o[2], o[3]);
   }
 }
 
@@ -161,8 +219,19 @@ extern "C" int bc4g_causal_conv(const void* in, int dtype, const float* in_bias,
                                                                        static_cast<T*>(state), seq_start, seq_slots,      \
                                                                        per_seq, channels, taps);                          \
   } while (0)
+  const bool pieces = dtype == kBF16 && channels % 8 == 0 && reinterpret_cast<uintptr_t>(in) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(out) % 16 == 0 && (taps == 1 || reinterpret_cast<uintptr_t>(state) % 16 == 0);
   if (dtype == kF32) BC4G_CONV(float);
-  else if (dtype == kBF16) BC4G_CONV(bf16_t);
+  else if (pieces) {
+    causal_conv_pieces_kernel<<<grid_for(total / 8), kBlock, 0, s>>>(
+        static_cast<const bf16_t*>(in), in_bias, w, out_bias, add_input, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(state),
+        row_seq, seq_start, seq_slots, total / 8, channels, taps);
+    if (taps > 1)
+      causal_conv_state_kernel<bf16_t><<<grid_for(per_seq), kBlock, 0, s>>>(static_cast<const bf16_t*>(in), in_bias,
+                                                                            static_cast<bf16_t*>(state), seq_start, seq_slots,
+                                                                            per_seq, channels, taps);
+  } else if (dtype == kBF16) BC4G_CONV(bf16_t);
   else return fail("causal_conv: unknown dtype %d", dtype);
 #undef BC4G_CONV
   return check_launch("causal_conv");

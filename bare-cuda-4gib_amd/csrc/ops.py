@@ -1185,15 +1185,16 @@ def _check_grouping(what: str, ctx, n_rows: int) -> None:
 def causal_conv(x: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Tensor], ctx, in_bias: Optional[torch.Tensor] = None,
                 out_bias: Optional[torch.Tensor] = None, add_input: bool = False) -> torch.Tensor:
     """A causal convolution over time on each channel of x [T, C], continued from every request's state
-    [slots, taps - 1, C] (x's dtype), which then receives the request's last taps - 1 inputs.  weight float32 [C, taps]
-    (its last column is the current token's); a row's input is x + in_bias; out_bias is added to the sum, and with
-    ``add_input`` x itself.  ``ctx``: the step's context (which rows belong to which request and slot)."""
+    [slots, taps - 1, C] (x's dtype), which then receives the request's last taps - 1 inputs.  weight float32
+    [taps, C]: by taps (a checkpoint's [C, taps] transposed; its last row is the current token's); a row's input is
+    x + in_bias; out_bias is added to the sum, and with ``add_input`` x itself.  ``ctx``: the step's context (which rows
+    belong to which request and slot)."""
     _dev("causal_conv", x, weight, state, in_bias, out_bias)
-    if x.dim() != 2 or weight.dim() != 2 or weight.shape[0] != x.shape[1]:
-        raise KernelError(f"causal_conv: x {tuple(x.shape)} and weight {tuple(weight.shape)} do not match")
+    if x.dim() != 2 or weight.dim() != 2 or weight.shape[1] != x.shape[1]:
+        raise KernelError(f"causal_conv: x {tuple(x.shape)} and weight {tuple(weight.shape)} (by taps) do not match")
     t, c = x.shape
-    taps = weight.shape[1]
-    _f32("causal_conv", "weight", weight, (c, taps))
+    taps = weight.shape[0]
+    _f32("causal_conv", "weight", weight, (taps, c))
     _f32("causal_conv", "in_bias", in_bias, (c,))
     _f32("causal_conv", "out_bias", out_bias, (c,))
     if taps > 1:

@@ -33,7 +33,7 @@ class CausalConv(Part):
         return out
 
     def bind(self, tensors, rt) -> None:
-        self.w = tensors["weight"].to(torch.float32).contiguous()
+        self.w = tensors["weight"].to(torch.float32).t().contiguous()      # by taps: neighbouring channels side by side
         self.b = tensors["bias"].to(torch.float32).contiguous() if self.bias else None
 
     def cache_spec(self):

@@ -44,7 +44,7 @@ class RGLRU(Part):
         self.w_y, self.w_x, self.w_o = (ops.StreamedWeight(tensors[n]) for n in ("y", "x", "o"))
         self.y_b, self.x_b, self.conv_b, self.lam = f32("y.b"), f32("x.b"), f32("conv.b"), f32("lam")
         self.ra_b, self.ri_b = f32("ra.b"), f32("ri.b")
-        self.conv_w = tensors["conv"].to(torch.float32).contiguous()
+        self.conv_w = tensors["conv"].to(torch.float32).t().contiguous()   # by taps
         # [block, 2 bs, bs]: both gates' matrices of a block in one product per block
         self.w_gates = torch.cat([tensors["ra"], tensors["ri"]], dim=1).contiguous()
         self.act_dtype = rt.act_dtype

@@ -260,7 +260,7 @@ def test_convolution_over_portions(dtype, taps):
             lens = [min(next(sizes), len(seqs[s]) - done[s]) for s in live]
             ctx = step_context(lens, [done[s] for s in live], [slots[s] for s in live])
             x = torch.cat([seqs[s][done[s]:done[s] + n] for s, n in zip(live, lens)]).to(dev)
-            out = ops.causal_conv(x, w.to(dev), st if taps > 1 else None, ctx, in_bias=b_in.to(dev), out_bias=b_out.to(dev),
+            out = ops.causal_conv(x, w.t().contiguous().to(dev), st if taps > 1 else None, ctx, in_bias=b_in.to(dev), out_bias=b_out.to(dev),
                                   add_input=add_input).cpu()
             at = 0
             for s, n in zip(live, lens):
