@@ -52,8 +52,12 @@ CONFIGS: Dict[str, dict] = {
         recurrent(32, 2, 3), recurrent(48, 3, 2, ff=40)]),                         # no attention: nothing is kept per token
     "U": dict(architecture="Mamenex", vocab=64, width=32, norm=dict(eps=1e-5), canon=dict(taps=5), layers=[
         latent(2, 8, 8, 8, 24, dims=8), latent(6, 4, 2, 4, 10, dims=2, ff=48)]),    # no recurrence
+    "V": dict(architecture="Mamenex", vocab=53, width=50, norm=dict(eps=1e-4), canon=dict(taps=6), layers=[
+        latent(3, 5, 6, 7, 9, dims=4, base=30.0, ff=35),                            # nothing a multiple of four
+        recurrent(30, 3, 7, ff=22),
+        latent(7, 3, 2, 5, 11, dims=2)]),
 }
-SEEDS = {"P": 11, "Q": 22, "R": 33, "S": 44, "T": 55, "U": 66}
+SEEDS = {"P": 11, "Q": 22, "R": 33, "S": 44, "T": 55, "U": 66, "V": 77}
 
 
 def tensors_for(config: dict, seed: int, query_factor: float = 3.0, sink_mean: float = 0.0) -> Dict[str, torch.Tensor]:

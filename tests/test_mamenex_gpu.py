@@ -21,7 +21,7 @@ pytestmark = pytest.mark.gpu
 # against float64 through up to four layers with peaked attention.  bfloat16: activations between kernels carry 8 bits; peaked attention multiplies what the layers before have
 # left (two keys that score alike change places), so the bfloat16 folders are drawn with smaller query weights.
 ROW_RMS = {"float32": 2e-5, "bfloat16": 5e-2}
-LENGTHS = {"P": [1, 2, 9, 70, 150], "Q": [3, 33, 64, 129], "R": [1, 17, 140], "S": [1, 5, 40, 131], "T": [1, 3, 90], "U": [2, 70]}
+LENGTHS = {"P": [1, 2, 9, 70, 150], "Q": [3, 33, 64, 129], "R": [1, 17, 140], "S": [1, 5, 40, 131], "T": [1, 3, 90], "U": [2, 70], "V": [1, 4, 75]}
 
 
 def close_rows(got, where, plain_logits, dtype, label, factor=1.0):
@@ -323,8 +323,9 @@ def test_recurrence_over_portions(dtype, blocks, width):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("sizes", [(3, 20, 12), (4, 48, 16), (20, 112, 16), (16, 512, 64)])
-@pytest.mark.parametrize("needle", [0, 5, 7, 8, 15, 16, 31, 32, 120, 198, 199])
+@pytest.mark.parametrize("sizes", [(3, 20, 12), (4, 48, 16), (20, 112, 16), (16, 512, 64), (8, 128, 64), (2, 256, 32), (33, 64, 64),
+                                   (5, 32, 0), (1, 700, 100)])
+@pytest.mark.parametrize("needle", [0, 7, 8, 31, 32, 120, 199])
 def test_latent_attention_finds_one_key_among_hundreds(dtype, needle, sizes):
     """200 cached rows in scattered pages of 8; one row, far back, at a page's border or the row's own, is made to
     score far above the others for one head: that head's output is that row's latent, the others' are not, and all
@@ -335,7 +336,8 @@ def test_latent_attention_finds_one_key_among_hundreds(dtype, needle, sizes):
     (H, rank, rot), dev, n, P, scale = sizes, "cuda:0", 200, 8, 0.3
     rows = (torch.randn(n, rank + rot) * 0.3).to(dtype)
     q = torch.randn(H, rank + rot)
-    rows[needle] = (q[1] / float(q[1] @ q[1]) * 14.0 / scale).to(dtype)        # its score for head 1: 14
+    mark = min(1, H - 1)
+    rows[needle] = (q[mark] / float(q[mark] @ q[mark]) * 14.0 / scale).to(dtype)        # its score for that head: 14
     sink = torch.randn(H) + 1.0
     pages = torch.randperm(40)[:n // P]
     tensor_cores = dtype == torch.bfloat16 and ops.attention_latent_mfma_takes(torch.empty(8, dtype=dtype, device=dev), rank, rot)
@@ -355,7 +357,7 @@ def test_latent_attention_finds_one_key_among_hundreds(dtype, needle, sizes):
                 w = plain.sink_softmax(s, float(sink[a]))
                 want = w @ rows[:pos + 1, :rank].double()
                 assert torch.allclose(got[k, a], want, atol=tol * float(want.abs().max()), rtol=tol), (needle, pos, a)
-                if a == 1 and needle <= pos:
+                if a == mark and needle <= pos:
                     assert float(w[needle]) > 0.9
 
 
