@@ -199,34 +199,43 @@ __global__ __launch_bounds__(256, 2) void latent_mfma_kernel(
   }
 }
 
-// The form for few rows (a decode step): a workgroup takes ONE tile of 16 (token, head) pairs and its four waves cut
-// the tile's work between them -- wave w the k-steps w, w + 4, ... of the scores (the partial scores are added up
-// through LDS, every wave in the same order, so all four hold the same bits and take the same maximum and sum) and
-// the blocks w, w + 4, ... of the latent for the output.  A wave then keeps a quarter of the queries and of the sums
-// in registers, and a tile's chain of LDS reads and matrix instructions is a quarter as long.
-template <int KS, int DB>
-__global__ __launch_bounds__(256) void latent_mfma_shared_kernel(
+// The form in which G waves cut one tile's work between them -- wave w of a tile the k-steps w, w + G, ... of the
+// scores (the partial scores are added up through LDS, every wave in the same order, so all hold the same bits and
+// take the same maximum and sum) and the blocks w, w + G, ... of the latent for the output.  A wave then keeps 1 / G of
+// the queries and of the sums in registers, and a tile's chain of LDS reads and matrix instructions is that much
+// shorter.  A workgroup has WAVES waves and WAVES / G tiles that follow each other.  Four waves on one tile serve a
+// decode step (a request's one row of up to sixteen heads is one tile).  (Eight waves on four tiles, two a tile, spill
+// nothing and were tried for prompts: no faster at 16 heads and slower at 32 than the form above -- its 90 KB of LDS
+// leave one workgroup a CU, whose eight waves then all wait at the same barriers, where two workgroups of the form
+// above stage and compute beside each other.)
+template <int KS, int DB, int G, int WAVES>
+__global__ __launch_bounds__(kWave * WAVES) void latent_mfma_shared_kernel(
     const float* __restrict__ q_lat, float* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     const bf16_t* __restrict__ cache, const float* __restrict__ sink, const int32_t* __restrict__ block_table,
     int table_stride, const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_ctx, int n_tokens, int heads,
     int rank, int dk, int page_tokens, int window, float scale, int hb, int tpt, int n_hg, int n_splits) {
   extern __shared__ uint4 tile[];                             // the tile, its latent part transposed, the partial scores
-  constexpr int KW = (KS + 3) / 4, DW = (DB + 3) / 4;         // k-steps and latent blocks of a wave
+  constexpr int KW = (KS + G - 1) / G, DW = (DB + G - 1) / G;   // k-steps and latent blocks of a wave
+  constexpr int TILES = WAVES / G, SUBS = 2 * WAVES;            // tiles of a workgroup; threads that stage one key
   const int s = blockIdx.y, z = blockIdx.z;
   const int tok0 = seq_start[s], n_tok = seq_start[s + 1] - tok0, cached = seq_ctx[s];
   const int n_tb = (n_tok + tpt - 1) / tpt, n_tiles = n_tb * n_hg;
-  const int my_tile = blockIdx.x;
-  if (my_tile >= n_tiles) return;
+  // (the grid's first workgroups take a request's last rows: their walks over the keys are the longest)
+  const int tile0 = (gridDim.x - 1 - blockIdx.x) * TILES;
+  if (tile0 >= n_tiles) return;                               // (the whole workgroup)
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  const int tb = my_tile / n_hg, hg = my_tile % n_hg;
+  const int my_tile = tile0 + wave / G, part_of_tile = wave % G;
+  const bool wave_live = my_tile < n_tiles;
+  const int tb = wave_live ? my_tile / n_hg : 0, hg = wave_live ? my_tile % n_hg : 0;
   const int c = lane % 16, g = lane / 16;
   const int tq = tb * tpt + c / hb, head = hg * hb + c % hb;
-  const bool q_live = c / hb < tpt && tq < n_tok && head < heads;
+  const bool q_live = wave_live && c / hb < tpt && tq < n_tok && head < heads;
   const int pos = cached + tq;
   const int32_t* table = block_table + static_cast<long>(s) * table_stride;
   const int cpr = dk / 8, pitch = cpr + 1;
-  const int last_pos = cached + min(n_tok, (tb + 1) * tpt) - 1;
-  const int first_pos = window > 0 ? max(0, cached + tb * tpt - window + 1) : 0;
+  const int tb_last = min(n_tb - 1, (tile0 + TILES - 1) / n_hg);
+  const int last_pos = cached + min(n_tok, (tb_last + 1) * tpt) - 1;
+  const int first_pos = window > 0 ? max(0, cached + (tile0 / n_hg) * tpt - window + 1) : 0;
   const int kt_begin = first_pos / kKeys, kt_end = last_pos / kKeys + 1;
   const int per = (kt_end - kt_begin + n_splits - 1) / n_splits;
   const int kt_lo = kt_begin + z * per, kt_hi = min(kt_end, kt_lo + per);
@@ -236,7 +245,7 @@ __global__ __launch_bounds__(256) void latent_mfma_shared_kernel(
     const float* qrow = q_lat + (static_cast<long>(tok0 + tq) * heads + head) * dk;
 #pragma unroll
     for (int i = 0; i < KW; ++i) {
-      const int ks = wave + 4 * i;
+      const int ks = part_of_tile + G * i;
       qf[i] = zero16();
       if (q_live && ks * 32 < dk) {
         const float4 a = *reinterpret_cast<const float4*>(qrow + ks * 32 + 8 * g);
@@ -253,8 +262,10 @@ __global__ __launch_bounds__(256) void latent_mfma_shared_kernel(
   uint16_t* vt = reinterpret_cast<uint16_t*>(tile + kKeys * pitch);
   float4* partial = reinterpret_cast<float4*>(reinterpret_cast<char*>(tile) + kKeys * pitch * 16 + ((rank * kVtPitch * 2 + 15) / 16) * 16);
 
-  constexpr int kPieces = (KS * 4 + 7) / 8;
-  const int st_key = threadIdx.x / 8, st_sub = threadIdx.x % 8;
+  // Staging: SUBS threads a key, each with every SUBS-th 16-byte piece of its row -- one look at the block table a
+  // thread and tile, all of a thread's loads asked for together.
+  constexpr int kPieces = (KS * 4 + SUBS - 1) / SUBS;
+  const int st_key = threadIdx.x / SUBS, st_sub = threadIdx.x % SUBS;
   uint4 stage[kPieces];
   for (int kt = kt_lo; kt < kt_hi; ++kt) {
     const int j0 = kt * kKeys;
@@ -265,13 +276,13 @@ __global__ __launch_bounds__(256) void latent_mfma_shared_kernel(
       if (there) src = cache + (static_cast<long>(table[j / page_tokens]) * page_tokens + j % page_tokens) * dk;
 #pragma unroll
       for (int p = 0; p < kPieces; ++p) {
-        const int part = st_sub + 8 * p;
+        const int part = st_sub + SUBS * p;
         stage[p] = there && part < cpr ? load16(src + part * 8) : zero16();
       }
     }
 #pragma unroll
     for (int p = 0; p < kPieces; ++p) {
-      const int part = st_sub + 8 * p;
+      const int part = st_sub + SUBS * p;
       if (part < cpr) tile[st_key * pitch + part] = stage[p];
       if (part * 8 < rank) {
         uint16_t* to = vt + part * 8 * kVtPitch + st_key;
@@ -285,56 +296,63 @@ __global__ __launch_bounds__(256) void latent_mfma_shared_kernel(
     }
     lds_barrier();
     floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    if (wave_live) {
 #pragma unroll
-    for (int i = 0; i < KW; ++i) {
-      const int ks = wave + 4 * i;
-      if (ks * 32 < dk) {
-        s0 = mfma_16x16x32(tile[c * pitch + ks * 4 + g], qf[i], s0);
-        s1 = mfma_16x16x32(tile[(16 + c) * pitch + ks * 4 + g], qf[i], s1);
+      for (int i = 0; i < KW; ++i) {
+        const int ks = part_of_tile + G * i;
+        if (ks * 32 < dk) {
+          s0 = mfma_16x16x32(tile[c * pitch + ks * 4 + g], qf[i], s0);
+          s1 = mfma_16x16x32(tile[(16 + c) * pitch + ks * 4 + g], qf[i], s1);
+        }
       }
     }
     partial[(wave * kWave + lane) * 2] = make_float4(s0[0], s0[1], s0[2], s0[3]);
     partial[(wave * kWave + lane) * 2 + 1] = make_float4(s1[0], s1[1], s1[2], s1[3]);
     lds_barrier();
-    float p[8];
+    if (wave_live) {
+      float p[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) p[i] = 0.f;
+      for (int i = 0; i < 8; ++i) p[i] = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {                             // (in this order in every wave)
-      const float4 a = partial[(w * kWave + lane) * 2], b = partial[(w * kWave + lane) * 2 + 1];
-      p[0] += a.x, p[1] += a.y, p[2] += a.z, p[3] += a.w, p[4] += b.x, p[5] += b.y, p[6] += b.z, p[7] += b.w;
-    }
-    float mx = -INFINITY;
+      for (int w = 0; w < G; ++w) {                           // (in this order in every wave of the tile)
+        const int from = ((wave / G) * G + w) * kWave + lane;
+        const float4 a = partial[from * 2], b = partial[from * 2 + 1];
+        p[0] += a.x, p[1] += a.y, p[2] += a.z, p[3] += a.w, p[4] += b.x, p[5] += b.y, p[6] += b.z, p[7] += b.w;
+      }
+      float mx = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int j = j0 + (i < 4 ? 0 : 16) + 4 * g + (i & 3);
-      const bool seen = q_live && j <= pos && (window == 0 || j > pos - window);
-      p[i] = seen ? p[i] * scale2 : -INFINITY;
-      mx = fmaxf(mx, p[i]);
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-    const float m_new = fmaxf(m, mx);
-    const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
-    float sum = 0.f;
+      for (int i = 0; i < 8; ++i) {
+        const int j = j0 + (i < 4 ? 0 : 16) + 4 * g + (i & 3);
+        const bool seen = q_live && j <= pos && (window == 0 || j > pos - window);
+        p[i] = seen ? p[i] * scale2 : -INFINITY;
+        mx = fmaxf(mx, p[i]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      const float m_new = fmaxf(m, mx);
+      const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
+      float sum = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      p[i] = p[i] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(p[i] - m_new);
-      sum += p[i];
-    }
-    l = l * alpha + sum;
-    m = m_new;
+      for (int i = 0; i < 8; ++i) {
+        p[i] = p[i] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(p[i] - m_new);
+        sum += p[i];
+      }
+      l = l * alpha + sum;
+      m = m_new;
+      if (__any(alpha != 1.f)) {
 #pragma unroll
-    for (int i = 0; i < DW; ++i) acc[i] *= alpha;
-    const uint4 pf = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
-    const uint16_t* col = vt + c * kVtPitch + 4 * g;
+        for (int i = 0; i < DW; ++i) acc[i] *= alpha;
+      }
+      const uint4 pf = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]), pack_bf16(p[6], p[7]));
+      const uint16_t* col = vt + c * kVtPitch + 4 * g;
 #pragma unroll
-    for (int i = 0; i < DW; ++i) {
-      const int db = wave + 4 * i;
-      if (db * 16 < rank) {
-        const uint2 lo = *reinterpret_cast<const uint2*>(col + db * 16 * kVtPitch);
-        const uint2 hi = *reinterpret_cast<const uint2*>(col + db * 16 * kVtPitch + 16);
-        acc[i] = mfma_16x16x32(make_uint4(lo.x, lo.y, hi.x, hi.y), pf, acc[i]);
+      for (int i = 0; i < DW; ++i) {
+        const int db = part_of_tile + G * i;
+        if (db * 16 < rank) {
+          const uint2 lo = *reinterpret_cast<const uint2*>(col + db * 16 * kVtPitch);
+          const uint2 hi = *reinterpret_cast<const uint2*>(col + db * 16 * kVtPitch + 16);
+          acc[i] = mfma_16x16x32(make_uint4(lo.x, lo.y, hi.x, hi.y), pf, acc[i]);
+        }
       }
     }
     lds_barrier();                                            // the tile has been read by everyone
@@ -349,14 +367,14 @@ __global__ __launch_bounds__(256) void latent_mfma_shared_kernel(
     if (sink) l += __builtin_amdgcn_exp2f(sink[head] * kLog2e - m);
     inv = 1.0f / l;
     o = out + row * rank;
-  } else if (wave == 0 && g == 0) {
+  } else if (part_of_tile == 0 && g == 0) {
     float* ml = part_ml + (static_cast<long>(z) * n_tokens * heads + row) * 2;
     ml[0] = m;
     ml[1] = l;
   }
 #pragma unroll
   for (int i = 0; i < DW; ++i) {
-    const int db = wave + 4 * i;
+    const int db = part_of_tile + G * i;
     if (db * 16 < rank)
       *reinterpret_cast<float4*>(o + db * 16 + 4 * g) = make_float4(acc[i][0] * inv, acc[i][1] * inv, acc[i][2] * inv, acc[i][3] * inv);
   }
@@ -433,26 +451,27 @@ extern "C" int bc4g_attention_latent_mfma(const float* q_lat, float* out, float*
   const int hb = heads < 16 ? heads : 16, tpt = 16 / hb, n_hg = ceil_div(heads, hb);
   const int most_tiles = ceil_div(most_tokens, tpt) * n_hg;
   BC4G_REQUIRE(n_seqs <= 65535 && n_splits <= 65535, "attention_latent_mfma: %d requests are beyond the grid limit", n_seqs);
-  // no request with four tiles (a decode step): a workgroup a tile, the waves cut the tile's work
-  const bool shared = most_tiles < 4;
-  dim3 grid(shared ? most_tiles : ceil_div(most_tiles, 4), n_seqs, n_splits);
+  // no request with four tiles (a decode step): a workgroup a tile, four waves on it; else four tiles a workgroup, a
+  // wave on each
+  const bool one_tile = most_tiles < 4;
+  dim3 grid(one_tile ? most_tiles : ceil_div(most_tiles, 4), n_seqs, n_splits);
   const size_t lds = static_cast<size_t>(kKeys) * (dk / 8 + 1) * 16 + (static_cast<size_t>(rank) * kVtPitch * 2 + 15) / 16 * 16 +
-                     (shared ? 4 * kWave * 32 : 0);
+                     (one_tile ? 4 * kWave * 32 : 0);
   const bf16_t* kc = static_cast<const bf16_t*>(cache);
   // (more than 64 KB of LDS a workgroup has to be asked for, once for a kernel: the most this kernel ever takes)
 #define BC4G_LATENT(KS, DB)                                                                                                 \
   static const hipError_t allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_mfma_kernel<KS, DB>),         \
                                                         hipFuncAttributeMaxDynamicSharedMemorySize,                          \
                                                         kKeys * (KS * 4 + 1) * 16 + DB * 16 * kVtPitch * 2);                 \
-  static const hipError_t allowed_shared = hipFuncSetAttribute(                                                              \
-      reinterpret_cast<const void*>(&latent_mfma_shared_kernel<KS, DB>), hipFuncAttributeMaxDynamicSharedMemorySize,         \
+  static const hipError_t allowed4 = hipFuncSetAttribute(                                                                    \
+      reinterpret_cast<const void*>(&latent_mfma_shared_kernel<KS, DB, 4, 4>), hipFuncAttributeMaxDynamicSharedMemorySize,   \
       kKeys * (KS * 4 + 1) * 16 + DB * 16 * kVtPitch * 2 + 4 * kWave * 32);                                                  \
-  BC4G_REQUIRE(allowed == hipSuccess && allowed_shared == hipSuccess,                                                        \
+  BC4G_REQUIRE(allowed == hipSuccess && allowed4 == hipSuccess,                                                              \
                "attention_latent_mfma: %zu bytes of LDS a workgroup are refused", lds);                                       \
-  if (shared)                                                                                                                 \
-    latent_mfma_shared_kernel<KS, DB><<<grid, 256, lds, s>>>(q_lat, out, part_o, part_ml, kc, sink, block_table, table_stride, \
-                                                             seq_start, seq_ctx, n_tokens, heads, rank, dk, page_tokens, window, \
-                                                             scale, hb, tpt, n_hg, n_splits);                                 \
+  if (one_tile)                                                                                                               \
+    latent_mfma_shared_kernel<KS, DB, 4, 4><<<grid, 4 * kWave, lds, s>>>(q_lat, out, part_o, part_ml, kc, sink, block_table,  \
+                                                                         table_stride, seq_start, seq_ctx, n_tokens, heads, rank, \
+                                                                         dk, page_tokens, window, scale, hb, tpt, n_hg, n_splits); \
   else                                                                                                                        \
     latent_mfma_kernel<KS, DB><<<grid, 256, lds, s>>>(q_lat, out, part_o, part_ml, kc, sink, block_table, table_stride, seq_start, \
                                                       seq_ctx, n_tokens, heads, rank, dk, page_tokens, window, scale, hb, tpt, n_hg, \
