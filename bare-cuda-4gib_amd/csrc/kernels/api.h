@@ -233,31 +233,34 @@ int bc4g_xielu(const void* in, void* out, int dtype, const float* pq, long total
 // by side; its last row is the current token's), where a row's input is in[row] + in_bias (rounded to the storage type) and
 // the inputs before a step's first row come from the request's state [slots, taps - 1, channels] (zero when the request
 // was admitted: zeros before the sequence).  Afterwards the state holds the request's last taps - 1 inputs.  The
-// step's rows are grouped by request: row_seq [T], seq_start [S + 1], seq_slots [S].  w, biases: float32.
+// step's rows are grouped by request: row_seq [T], seq_start [S + 1], seq_slots [S].  w, biases: float32.  in_row: elements
+// from one row of in to the next (in may be a part of wider rows).
 int bc4g_causal_conv(const void* in, int dtype, const float* in_bias, const float* w, const float* out_bias, int add_input,
                      void* out, void* state, const int32_t* row_seq, const int32_t* seq_start, const int32_t* seq_slots,
-                     int n_rows, int n_seqs, int channels, int taps, void* stream);
+                     int n_rows, int n_seqs, int channels, int taps, long in_row, void* stream);
 // The real-gated linear recurrent unit over a step's rows.  pre [T, blocks, 2 bs] (float32): the gates' sums of
 // every block, Ra u_b then Ri u_b (a product per block: bc4g_heads_gemm); u, y [T, width]; decay a = exp(-8
 // sigmoid(Ra u + ra_b) softplus(lam)), S_t = a S_(t-1) + sqrt(1 - a^2) sigmoid(Ri u + ri_b) u along every request's
 // rows, from state [slots, width] (float32) and back into it; out[t] = S_t * gelu_tanh(y[t] + y_bias).  A request's
 // rows are walked in chunks of 64 by threads of their own: chunk_a, chunk_b [S, ceil(most_rows / 64), width] and
-// before [S, width] are scratch (float32); most_rows: the most rows one request brings.
+// before [S, width] are scratch (float32); most_rows: the most rows one request brings; y_row: elements from one row of y
+// to the next.
 int bc4g_rglru_scan(const float* pre, const void* u, const void* y, int dtype, const float* ra_b, const float* ri_b,
                     const float* lam, const float* y_bias, void* out, float* state, float* chunk_a, float* chunk_b,
                     float* before, const int32_t* seq_start, const int32_t* seq_slots, int n_rows, int n_seqs, int most_rows,
-                    int width, int blocks, void* stream);
+                    int width, int blocks, long y_row, void* stream);
 
 // Latent attention (attention_latent.hip).  q [T, heads, plain + rot] and dkv [T, rank + rot] as projected; the row's
 // cache slot (slot_map[t] = page * page_tokens + offset; cache [pages, page_tokens, rank + rot]; null: nothing is
 // written) receives [rmsnorm(dkv[:rank]) * g | rotate(dkv[rank:])], and q_lat [T, heads, rank + rot] (float32) the
 // rotated part of every head's query in its last rot numbers.  Elements 2i and 2i + 1 of the first `dims` numbers of
 // a rotated part turn by position * base^(-2i / dims): angles [T, dims / 2, 2] holds every row's cosines and sines
-// (bc4g_latent_angles makes it, the angles worked out in double: once a step for all layers of one rotation).
+// (bc4g_latent_angles makes it, the angles worked out in double: once a step for all layers of one rotation).  q_row,
+// dkv_row: elements from one row to the next (q and dkv may be parts of one product's rows).
 int bc4g_latent_angles(const int32_t* positions, float* table, int n_rows, int dims, float base, void* stream);
 int bc4g_latent_prepare(const void* q, const void* dkv, int dtype, const float* g, float eps, const float* angles,
                         const int32_t* slot_map, void* cache, float* q_lat, int n_rows, int heads, int plain, int rot,
-                        int rank, int dims, void* stream);
+                        int rank, int dims, long q_row, long dkv_row, void* stream);
 // out[t, h, :n] = w[h] a[t, h, :k] for every head: a at a + t * a_row + h * a_head, out likewise, w [heads, n, k].
 int bc4g_heads_gemm(const void* a, int a_dtype, long a_row, long a_head, const void* w, int w_dtype, void* out, int out_dtype,
                     long o_row, long o_head, int m, int n, int k, int heads, void* stream);

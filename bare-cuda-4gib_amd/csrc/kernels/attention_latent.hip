@@ -44,19 +44,20 @@ __global__ void latent_angles_kernel(const int32_t* __restrict__ positions, floa
   }
 }
 
-// One workgroup a row.  q: [T, heads, plain + rot] (as projected); dkv: [T, rank + rot]; q_lat: [T, heads, rank + rot]
+// One workgroup a row.  q: [T, heads, plain + rot] (as projected); dkv: [T, rank + rot] (rows q_row and dkv_row elements
+// apart: both may be parts of one product's rows); q_lat: [T, heads, rank + rot]
 // float, of which this kernel writes the last rot of every head; the row's cache slot receives [normed latent | rotated
 // key part].  Neighbouring elements 2i and 2i + 1 of the first `dims` of a rotated part are a pair; the rest passes.
 template <typename T>
 __global__ __launch_bounds__(kPrepBlock) void latent_prepare_kernel(
     const T* __restrict__ q, const T* __restrict__ dkv, const float* __restrict__ g, float eps,
     const float* __restrict__ angles, const int32_t* __restrict__ slot_map, T* __restrict__ cache,
-    float* __restrict__ q_lat, int heads, int plain, int rot, int rank, int dims) {
+    float* __restrict__ q_lat, int heads, int plain, int rot, int rank, int dims, long q_row, long dkv_row) {
   __shared__ float scratch[16];
   extern __shared__ float cs[];                     // [dims / 2][2]: the row's cosines and sines
   const long row = blockIdx.x;
   for (int i = threadIdx.x; i < dims; i += kPrepBlock) cs[i] = angles[row * dims + i];
-  const T* lat = dkv + row * (rank + rot);
+  const T* lat = dkv + row * dkv_row;
   float ss = 0.f;
   for (int i = threadIdx.x; i < rank; i += kPrepBlock) {
     const float v = to_float(lat[i]);
@@ -75,7 +76,7 @@ __global__ __launch_bounds__(kPrepBlock) void latent_prepare_kernel(
       to[rank + i] = from_float<T>(v);
     }
   }
-  const T* qr = q + row * heads * (plain + rot);
+  const T* qr = q + row * q_row;
   float* ql = q_lat + row * heads * (rank + rot);
   for (int e = threadIdx.x; e < heads * rot; e += kPrepBlock) {
     const int h = e / rot, i = e % rot;
@@ -313,23 +314,25 @@ extern "C" int bc4g_latent_angles(const int32_t* positions, float* table, int n_
 
 extern "C" int bc4g_latent_prepare(const void* q, const void* dkv, int dtype, const float* g, float eps,
                                    const float* angles, const int32_t* slot_map, void* cache, float* q_lat,
-                                   int n_rows, int heads, int plain, int rot, int rank, int dims, void* stream) {
+                                   int n_rows, int heads, int plain, int rot, int rank, int dims, long q_row, long dkv_row,
+                                   void* stream) {
   BC4G_REQUIRE(n_rows >= 0 && heads > 0 && plain >= 0 && rot >= 0 && rank > 0, "latent_prepare: bad sizes T=%d heads=%d "
                "plain=%d rot=%d rank=%d", n_rows, heads, plain, rot, rank);
   BC4G_REQUIRE(dims >= 0 && dims % 2 == 0 && dims <= rot && dims <= 8192,
                "latent_prepare: %d rotated dimensions of %d (even, at most the rotated part)", dims, rot);
   BC4G_REQUIRE(q && dkv && g && (angles || dims == 0) && q_lat && (!cache || slot_map), "latent_prepare: a tensor is missing");
+  BC4G_REQUIRE(q_row >= static_cast<long>(heads) * (plain + rot) && dkv_row >= rank + rot, "latent_prepare: rows shorter than their parts");
   if (n_rows == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const size_t lds = static_cast<size_t>(dims > 0 ? dims : 2) * sizeof(float);
   if (dtype == kF32)
     latent_prepare_kernel<float><<<n_rows, kPrepBlock, lds, s>>>(static_cast<const float*>(q), static_cast<const float*>(dkv), g,
                                                                  eps, angles, slot_map, static_cast<float*>(cache), q_lat,
-                                                                 heads, plain, rot, rank, dims);
+                                                                 heads, plain, rot, rank, dims, q_row, dkv_row);
   else if (dtype == kBF16)
     latent_prepare_kernel<bf16_t><<<n_rows, kPrepBlock, lds, s>>>(static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(dkv),
                                                                   g, eps, angles, slot_map, static_cast<bf16_t*>(cache),
-                                                                  q_lat, heads, plain, rot, rank, dims);
+                                                                  q_lat, heads, plain, rot, rank, dims, q_row, dkv_row);
   else return fail("latent_prepare: unknown dtype %d", dtype);
   return check_launch("latent_prepare");
 }

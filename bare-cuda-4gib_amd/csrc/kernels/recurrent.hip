@@ -22,8 +22,8 @@ int grid_for(long total) {
 // The input of row `at` of a request, as it is kept: with the input's bias added and rounded to the storage type
 // (what the state holds of earlier steps is rounded so too: the result does not depend on where a prompt was cut).
 template <typename T>
-__device__ inline float conv_input(const T* in, const float* in_bias, long at, int c, int channels) {
-  const float v = to_float(in[at * channels + c]);
+__device__ inline float conv_input(const T* in, const float* in_bias, long at, int c, long in_row) {
+  const float v = to_float(in[at * in_row + c]);
   return in_bias ? to_float(from_float<T>(v + in_bias[c])) : v;
 }
 
@@ -33,7 +33,7 @@ __global__ void causal_conv_kernel(const T* __restrict__ in, const float* __rest
                                    const float* __restrict__ w, const float* __restrict__ out_bias, int add_input,
                                    T* __restrict__ out, const T* __restrict__ state, const int32_t* __restrict__ row_seq,
                                    const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slots,
-                                   long total, int channels, int taps) {
+                                   long total, int channels, int taps, long in_row) {
   const long stride = static_cast<long>(blockDim.x) * gridDim.x;
   for (long idx = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; idx < total; idx += stride) {
     const int c = static_cast<int>(idx % channels);
@@ -45,11 +45,11 @@ __global__ void causal_conv_kernel(const T* __restrict__ in, const float* __rest
     float acc = out_bias ? out_bias[c] : 0.f;
     for (int j = 0; j < taps; ++j) {
       const int src = local - (taps - 1) + j;
-      const float v = src >= 0 ? conv_input(in, in_bias, start + src, c, channels)
+      const float v = src >= 0 ? conv_input(in, in_bias, start + src, c, in_row)
                                : to_float(tail[static_cast<long>(taps - 1 + src) * channels + c]);
       acc = fmaf(w[static_cast<long>(j) * channels + c], v, acc);
     }
-    if (add_input) acc += to_float(in[idx]);
+    if (add_input) acc += to_float(in[t * in_row + c]);
     out[idx] = from_float<T>(acc);
   }
 }
@@ -66,7 +66,7 @@ __global__ void causal_conv_pieces_kernel(const bf16_t* __restrict__ in, const f
                                           const float* __restrict__ w, const float* __restrict__ out_bias, int add_input,
                                           bf16_t* __restrict__ out, const bf16_t* __restrict__ state,
                                           const int32_t* __restrict__ row_seq, const int32_t* __restrict__ seq_start,
-                                          const int32_t* __restrict__ seq_slots, long total, int channels, int taps) {
+                                          const int32_t* __restrict__ seq_slots, long total, int channels, int taps, long in_row) {
   const int pieces = channels / 8;
   const long stride = static_cast<long>(blockDim.x) * gridDim.x;
   for (long idx = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; idx < total; idx += stride) {
@@ -83,7 +83,7 @@ __global__ void causal_conv_pieces_kernel(const bf16_t* __restrict__ in, const f
       const int src = local - (taps - 1) + j;
       float v[8];
       if (src >= 0) {
-        widen8(load16(in + (start + src) * channels + c0), v);
+        widen8(load16(in + (start + src) * in_row + c0), v);
         if (in_bias) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) v[e] = to_float(from_float<bf16_t>(v[e] + bias[e]));      // as the tail keeps it
@@ -99,7 +99,7 @@ __global__ void causal_conv_pieces_kernel(const bf16_t* __restrict__ in, const f
     }
     if (add_input) {
       float v[8];
-      widen8(load16(in + t * channels + c0), v);
+      widen8(load16(in + t * in_row + c0), v);
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[e] += v[e];
     }
@@ -116,7 +116,7 @@ __global__ void causal_conv_pieces_kernel(const bf16_t* __restrict__ in, const f
 template <typename T>
 __global__ void causal_conv_state_kernel(const T* __restrict__ in, const float* __restrict__ in_bias, T* __restrict__ state,
                                          const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slots,
-                                         long total, int channels, int taps) {
+                                         long total, int channels, int taps, long in_row) {
   const long stride = static_cast<long>(blockDim.x) * gridDim.x;
   for (long idx = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; idx < total; idx += stride) {
     const int c = static_cast<int>(idx % channels);
@@ -127,7 +127,7 @@ __global__ void causal_conv_state_kernel(const T* __restrict__ in, const float* 
     for (int i = 0; i < taps - 1; ++i) {
       const int src = n - (taps - 1) + i;
       tail[static_cast<long>(i) * channels + c] =
-          src >= 0 ? from_float<T>(conv_input(in, in_bias, start + src, c, channels))
+          src >= 0 ? from_float<T>(conv_input(in, in_bias, start + src, c, in_row))
                    : tail[static_cast<long>(i + n) * channels + c];
     }
   }
@@ -159,7 +159,8 @@ __global__ __launch_bounds__(kWave) void rglru_chunks_kernel(
     const float* __restrict__ pre, const T* __restrict__ u, const T* __restrict__ y, const float* __restrict__ ra_b,
     const float* __restrict__ ri_b, const float* __restrict__ lam, const float* __restrict__ y_bias, T* __restrict__ out,
     float* __restrict__ state, float* __restrict__ chunk_a, float* __restrict__ chunk_b, float* __restrict__ before,
-    const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slots, int width, int bs, int most_chunks) {
+    const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slots, int width, int bs, int most_chunks,
+    long y_row) {
   const int ch = blockIdx.x * kWave + threadIdx.x, chunk = blockIdx.y, s = blockIdx.z;
   const long start = seq_start[s], end = seq_start[s + 1];
   const long lo = start + static_cast<long>(chunk) * kChunk, hi = lo + kChunk < end ? lo + kChunk : end;
@@ -188,7 +189,7 @@ __global__ __launch_bounds__(kWave) void rglru_chunks_kernel(
       float a, x;
       decay_and_drive(pa[t * 2 * width], pa[t * 2 * width + bs], to_float(u[t * width + ch]), ba, bi, sp, &a, &x);
       st = fmaf(a, st, x);
-      out[t * width + ch] = from_float<T>(st * gelu_tanh_f(to_float(y[t * width + ch]) + yb));
+      out[t * width + ch] = from_float<T>(st * gelu_tanh_f(to_float(y[t * y_row + ch]) + yb));
     }
     if (hi == end) *slot = st;
   }
@@ -201,11 +202,12 @@ using namespace bc4g;
 
 extern "C" int bc4g_causal_conv(const void* in, int dtype, const float* in_bias, const float* w, const float* out_bias,
                                 int add_input, void* out, void* state, const int32_t* row_seq, const int32_t* seq_start,
-                                const int32_t* seq_slots, int n_rows, int n_seqs, int channels, int taps, void* stream) {
+                                const int32_t* seq_slots, int n_rows, int n_seqs, int channels, int taps, long in_row,
+                                void* stream) {
   BC4G_REQUIRE(n_rows >= 0 && n_seqs >= 0 && channels > 0 && taps >= 1, "causal_conv: bad sizes T=%d S=%d C=%d taps=%d",
                n_rows, n_seqs, channels, taps);
-  BC4G_REQUIRE(in && w && out && in != out && row_seq && seq_start && seq_slots && (taps == 1 || state),
-               "causal_conv: a tensor is missing (or the output is the input)");
+  BC4G_REQUIRE(in && w && out && in != out && row_seq && seq_start && seq_slots && (taps == 1 || state) && in_row >= channels,
+               "causal_conv: a tensor is missing (or the output is the input, or the input's rows are shorter than the channels)");
   if (n_rows == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const long total = static_cast<long>(n_rows) * channels, per_seq = static_cast<long>(n_seqs) * channels;
@@ -213,24 +215,24 @@ extern "C" int bc4g_causal_conv(const void* in, int dtype, const float* in_bias,
   do {                                                                                                                    \
     causal_conv_kernel<T><<<grid_for(total), kBlock, 0, s>>>(static_cast<const T*>(in), in_bias, w, out_bias, add_input, \
                                                              static_cast<T*>(out), static_cast<const T*>(state), row_seq, \
-                                                             seq_start, seq_slots, total, channels, taps);                \
+                                                             seq_start, seq_slots, total, channels, taps, in_row);        \
     if (taps > 1)                                                                                                         \
       causal_conv_state_kernel<T><<<grid_for(per_seq), kBlock, 0, s>>>(static_cast<const T*>(in), in_bias,                \
                                                                        static_cast<T*>(state), seq_start, seq_slots,      \
-                                                                       per_seq, channels, taps);                          \
+                                                                       per_seq, channels, taps, in_row);                  \
   } while (0)
-  const bool pieces = dtype == kBF16 && channels % 8 == 0 && reinterpret_cast<uintptr_t>(in) % 16 == 0 &&
+  const bool pieces = dtype == kBF16 && channels % 8 == 0 && in_row % 8 == 0 && reinterpret_cast<uintptr_t>(in) % 16 == 0 &&
                       reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
                       reinterpret_cast<uintptr_t>(out) % 16 == 0 && (taps == 1 || reinterpret_cast<uintptr_t>(state) % 16 == 0);
   if (dtype == kF32) BC4G_CONV(float);
   else if (pieces) {
     causal_conv_pieces_kernel<<<grid_for(total / 8), kBlock, 0, s>>>(
         static_cast<const bf16_t*>(in), in_bias, w, out_bias, add_input, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(state),
-        row_seq, seq_start, seq_slots, total / 8, channels, taps);
+        row_seq, seq_start, seq_slots, total / 8, channels, taps, in_row);
     if (taps > 1)
       causal_conv_state_kernel<bf16_t><<<grid_for(per_seq), kBlock, 0, s>>>(static_cast<const bf16_t*>(in), in_bias,
                                                                             static_cast<bf16_t*>(state), seq_start, seq_slots,
-                                                                            per_seq, channels, taps);
+                                                                            per_seq, channels, taps, in_row);
   } else if (dtype == kBF16) BC4G_CONV(bf16_t);
   else return fail("causal_conv: unknown dtype %d", dtype);
 #undef BC4G_CONV
@@ -240,11 +242,11 @@ extern "C" int bc4g_causal_conv(const void* in, int dtype, const float* in_bias,
 extern "C" int bc4g_rglru_scan(const float* pre, const void* u, const void* y, int dtype, const float* ra_b, const float* ri_b,
                                const float* lam, const float* y_bias, void* out, float* state, float* chunk_a, float* chunk_b,
                                float* before, const int32_t* seq_start, const int32_t* seq_slots, int n_rows, int n_seqs,
-                               int most_rows, int width, int blocks, void* stream) {
+                               int most_rows, int width, int blocks, long y_row, void* stream) {
   BC4G_REQUIRE(n_rows >= 0 && n_seqs >= 0 && width > 0 && blocks > 0 && width % blocks == 0 && n_seqs <= 65535 && most_rows >= 0,
                "rglru_scan: bad sizes T=%d S=%d W=%d blocks=%d", n_rows, n_seqs, width, blocks);
-  BC4G_REQUIRE(pre && u && y && ra_b && ri_b && lam && out && state && chunk_a && chunk_b && before && seq_start && seq_slots,
-               "rglru_scan: a tensor is missing");
+  BC4G_REQUIRE(pre && u && y && ra_b && ri_b && lam && out && state && chunk_a && chunk_b && before && seq_start && seq_slots &&
+               y_row >= width, "rglru_scan: a tensor is missing (or y's rows are shorter than the width)");
   if (n_rows == 0 || n_seqs == 0 || most_rows == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int most_chunks = ceil_div(most_rows, kChunk);
@@ -254,10 +256,10 @@ extern "C" int bc4g_rglru_scan(const float* pre, const void* u, const void* y, i
   do {                                                                                                                          \
     rglru_chunks_kernel<T, false><<<grid, kWave, 0, s>>>(pre, static_cast<const T*>(u), static_cast<const T*>(y), ra_b, ri_b,  \
                                                          lam, y_bias, static_cast<T*>(out), state, chunk_a, chunk_b, before,   \
-                                                         seq_start, seq_slots, width, width / blocks, most_chunks);            \
+                                                         seq_start, seq_slots, width, width / blocks, most_chunks, y_row);     \
     rglru_chunks_kernel<T, true><<<grid, kWave, 0, s>>>(pre, static_cast<const T*>(u), static_cast<const T*>(y), ra_b, ri_b,   \
                                                         lam, y_bias, static_cast<T*>(out), state, chunk_a, chunk_b, before,    \
-                                                        seq_start, seq_slots, width, width / blocks, most_chunks);             \
+                                                        seq_start, seq_slots, width, width / blocks, most_chunks, y_row);      \
   } while (0)
   if (dtype == kF32) BC4G_SCAN(float);
   else if (dtype == kBF16) BC4G_SCAN(bf16_t);

@@ -1174,6 +1174,15 @@ def xielu(z: torch.Tensor, pq: torch.Tensor, out: Optional[torch.Tensor] = None)
     return out
 
 
+def _rows_of(what: str, name: str, t: torch.Tensor) -> int:
+    """The row stride of a [T, C] tensor on the GPU whose rows may be parts of wider rows (columns of one product's
+    output): the elements of a row lie side by side."""
+    if not t.is_cuda or t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1) or t.stride(0) < t.shape[1]:
+        raise KernelError(f"{what}: {name} must be [T, C] on the GPU with a row's elements side by side, got strides {t.stride()} "
+                          f"for shape {tuple(t.shape)} on {t.device}")
+    return t.stride(0)
+
+
 def _check_grouping(what: str, ctx, n_rows: int) -> None:
     if ctx.n_tokens != n_rows:
         raise KernelError(f"{what}: {n_rows} rows for a step of {ctx.n_tokens}")
@@ -1189,7 +1198,8 @@ def causal_conv(x: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Ten
     [taps, C]: by taps (a checkpoint's [C, taps] transposed; its last row is the current token's); a row's input is
     x + in_bias; out_bias is added to the sum, and with ``add_input`` x itself.  ``ctx``: the step's context (which rows
     belong to which request and slot)."""
-    _dev("causal_conv", x, weight, state, in_bias, out_bias)
+    _dev("causal_conv", weight, state, in_bias, out_bias)
+    in_row = _rows_of("causal_conv", "x", x)             # (x may be a part of one product's wider rows)
     if x.dim() != 2 or weight.dim() != 2 or weight.shape[1] != x.shape[1]:
         raise KernelError(f"causal_conv: x {tuple(x.shape)} and weight {tuple(weight.shape)} (by taps) do not match")
     t, c = x.shape
@@ -1203,10 +1213,10 @@ def causal_conv(x: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Ten
         if max(ctx.seq_slots, default=0) >= state.shape[0]:
             raise KernelError(f"causal_conv: a slot beyond the state's {state.shape[0]}")
     _check_grouping("causal_conv", ctx, t)
-    out = torch.empty_like(x)
+    out = torch.empty((t, c), dtype=x.dtype, device=x.device)
     library.call("bc4g_causal_conv", _ptr(x), _code(x, "causal_conv"), _ptr(in_bias), _ptr(weight), _ptr(out_bias),
                  1 if add_input else 0, _ptr(out), _ptr(state), _ptr(ctx.row_seq), _ptr(ctx.seq_start_dev),
-                 _ptr(ctx.seq_slots_dev), t, ctx.n_seqs, c, taps, _stream(),
+                 _ptr(ctx.seq_slots_dev), t, ctx.n_seqs, c, taps, in_row, _stream(),
                  cost=lambda: (2.0 * t * c * taps, 2 * t * c * x.element_size()))
     return out
 
@@ -1220,7 +1230,8 @@ def rglru(u: torch.Tensor, y: torch.Tensor, w_gates: torch.Tensor, ra_b: torch.T
     the matrix of the recurrence gate, then that of the input gate, each [out, in]); biases and lam float32 [W]; state
     float32 [slots, W].  The gates' sums are a product per block (float32 out), the gates, the decay and the state
     float32.  Returns S_t * gelu_tanh(y + y_bias) in u's dtype."""
-    _dev("rglru", u, y, w_gates, ra_b, ri_b, lam, y_bias, state)
+    _dev("rglru", u, w_gates, ra_b, ri_b, lam, y_bias, state)
+    y_row = _rows_of("rglru", "y", y)                     # (y may be a part of one product's wider rows)
     if u.dim() != 2 or y.shape != u.shape or y.dtype != u.dtype:
         raise KernelError(f"rglru: u and y must be alike [T, W], got {tuple(u.shape)} and {tuple(y.shape)}")
     t, w = u.shape
@@ -1240,7 +1251,7 @@ def rglru(u: torch.Tensor, y: torch.Tensor, w_gates: torch.Tensor, ra_b: torch.T
     out = torch.empty_like(u)
     library.call("bc4g_rglru_scan", _ptr(pre), _ptr(u), _ptr(y), _code(y, "rglru"), _ptr(ra_b), _ptr(ri_b), _ptr(lam), _ptr(y_bias),
                  _ptr(out), _ptr(state), _ptr(scratch[:chunks]), _ptr(scratch[chunks:2 * chunks]), _ptr(scratch[2 * chunks]),
-                 _ptr(ctx.seq_start_dev), _ptr(ctx.seq_slots_dev), t, ctx.n_seqs, most, w, blocks, _stream(),
+                 _ptr(ctx.seq_start_dev), _ptr(ctx.seq_slots_dev), t, ctx.n_seqs, most, w, blocks, y_row, _stream(),
                  cost=lambda: (40.0 * t * w, t * w * (16 + 5 * u.element_size())))
     return out
 
@@ -1292,7 +1303,8 @@ def latent_prepare(q: torch.Tensor, dkv: torch.Tensor, g: torch.Tensor, eps: flo
     """Writes [rmsnorm(dkv[:, :rank]) * g | rotate(dkv[:, rank:])] into every row's cache slot (``cache`` None: nowhere)
     and every head's rotated query part into q_lat[:, h, rank:].  ``angles``: latent_angles of the rows (None where
     nothing is rotated, dims 0)."""
-    _dev("latent_prepare", q, dkv, g, angles, slot_map, cache, q_lat)
+    _dev("latent_prepare", g, angles, slot_map, cache, q_lat)
+    q_row, dkv_row = _rows_of("latent_prepare", "q", q), _rows_of("latent_prepare", "dkv", dkv)   # (parts of one product's rows)
     t = q.shape[0]
     if q.dtype != dkv.dtype or tuple(q.shape) != (t, heads * (plain + rot)) or tuple(dkv.shape) != (t, rank + rot):
         raise KernelError(f"latent_prepare: q {tuple(q.shape)} / dkv {tuple(dkv.shape)} do not fit heads={heads} plain={plain} rot={rot} rank={rank}")
@@ -1306,18 +1318,20 @@ def latent_prepare(q: torch.Tensor, dkv: torch.Tensor, g: torch.Tensor, eps: flo
         _i32("latent_prepare", "slot_map", slot_map, t)
     library.call("bc4g_latent_prepare", _ptr(q), _ptr(dkv), _code(q, "latent_prepare"), _ptr(g), float(eps),
                  _ptr(angles) if dims else None, _ptr(slot_map) if cache is not None else None, _ptr(cache), _ptr(q_lat), t, heads,
-                 plain, rot, rank, int(dims), _stream(), cost=lambda: (4.0 * t * (rank + (heads + 1) * rot), t * (q.element_size() * (heads + 2) * rot + 2 * rank * q.element_size())))
+                 plain, rot, rank, int(dims), q_row, dkv_row, _stream(), cost=lambda: (4.0 * t * (rank + (heads + 1) * rot), t * (q.element_size() * (heads + 2) * rot + 2 * rank * q.element_size())))
 
 
 def heads_gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, k: int, n: int) -> None:
     """out[t, h, :n] = w[h] a[t, h, :k] for a [T, heads, >= k], w [heads, n, k], out [T, heads, >= n] (the last
     dimensions may be longer than k and n: parts of wider rows)."""
-    _dev("heads_gemm", a, w, out)
+    _dev("heads_gemm", w, out)
     if a.dim() != 3 or out.dim() != 3 or w.dim() != 3 or a.shape[:2] != out.shape[:2] or a.shape[2] < k or out.shape[2] < n \
             or tuple(w.shape) != (a.shape[1], n, k):
         raise KernelError(f"heads_gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit k={k}, n={n}")
+    if not a.is_cuda or a.stride(2) != 1 or a.stride(1) < k or a.stride(0) < a.stride(1):      # (a's rows may be parts of wider rows)
+        raise KernelError(f"heads_gemm: a must lie on the GPU with a head's elements side by side, got strides {a.stride()}")
     t, heads = a.shape[0], a.shape[1]
-    library.call("bc4g_heads_gemm", _ptr(a), _code(a, "heads_gemm"), heads * a.shape[2], a.shape[2], _ptr(w), _code(w, "heads_gemm"),
+    library.call("bc4g_heads_gemm", _ptr(a), _code(a, "heads_gemm"), a.stride(0), a.stride(1), _ptr(w), _code(w, "heads_gemm"),
                  _ptr(out), _code(out, "heads_gemm"), heads * out.shape[2], out.shape[2], t, n, k, heads, _stream(),
                  cost=lambda: (2.0 * t * heads * n * k, heads * n * k * w.element_size() + t * heads * (k * a.element_size() + n * out.element_size())))
 

@@ -56,8 +56,8 @@ class LatentAttention(Part):
 
     def bind(self, tensors, rt) -> None:
         H = self.heads
-        self.w_q = ops.StreamedWeight(tensors["q"])
-        self.w_dkv = ops.StreamedWeight(tensors["dkv"])
+        # one product for the queries and the latent: their rows one after the other
+        self.w_qd = ops.StreamedWeight(torch.cat([tensors["q"], tensors["dkv"]], dim=0).contiguous())
         self.w_o = ops.StreamedWeight(tensors["o"])
         self.g = tensors["dkv.norm"].to(torch.float32).contiguous()
         # [heads, rank, dim]: the keys' up-projection as it is applied to the query
@@ -78,8 +78,9 @@ class LatentAttention(Part):
 
     def forward(self, h, ctx, cache, residual, writes: bool = True) -> None:
         H, rank, rot, t = self.heads, self.kv_rank, self.rot_dim, h.shape[0]
-        q = linear(h, self.w_q, out_dtype=self.act_dtype)
-        dkv = linear(h, self.w_dkv, out_dtype=self.act_dtype)
+        n_q = H * (self.dim + rot)
+        qd = linear(h, self.w_qd, out_dtype=self.act_dtype)
+        q, dkv = qd[:, :n_q], qd[:, n_q:]
         q_lat = torch.empty((t, H, rank + rot), dtype=torch.float32, device=q.device)
         angles = None
         if self.rot_dims:                 # the same in every layer that rotates alike: a table made once a step
@@ -87,7 +88,7 @@ class LatentAttention(Part):
                                 lambda: ops.latent_angles(ctx.positions, self.rot_dims, self.rot_base))
         ops.latent_prepare(q, dkv, self.g, self.eps, angles, ctx.slot_maps[cache.group] if writes else None,
                            cache.latent if writes else None, q_lat, H, self.dim, rot, rank, self.rot_dims)
-        ops.heads_gemm(q.view(t, H, self.dim + rot), self.uk_t, q_lat, k=self.dim, n=rank)
+        ops.heads_gemm(q.unflatten(1, (H, self.dim + rot)), self.uk_t, q_lat, k=self.dim, n=rank)
         mixed = ops.attention_latent(q_lat, cache.latent, self.sinks, ctx.block_tables[cache.group], ctx, H, rank, rot,
                                      cache.page_tokens, self.window, self.scale)
         o = torch.empty((t, H, self.vdim), dtype=self.act_dtype, device=q.device)

@@ -41,7 +41,9 @@ class RGLRU(Part):
 
     def bind(self, tensors, rt) -> None:
         f32 = lambda name: tensors[name].to(torch.float32).reshape(-1).contiguous()      # noqa: E731
-        self.w_y, self.w_x, self.w_o = (ops.StreamedWeight(tensors[n]) for n in ("y", "x", "o"))
+        # one product for both branches: the gated branch's rows, then the recurrent one's
+        self.w_yx = ops.StreamedWeight(torch.cat([tensors["y"], tensors["x"]], dim=0).contiguous())
+        self.w_o = ops.StreamedWeight(tensors["o"])
         self.y_b, self.x_b, self.conv_b, self.lam = f32("y.b"), f32("x.b"), f32("conv.b"), f32("lam")
         self.ra_b, self.ri_b = f32("ra.b"), f32("ri.b")
         self.conv_w = tensors["conv"].to(torch.float32).t().contiguous()   # by taps
@@ -50,8 +52,8 @@ class RGLRU(Part):
         self.act_dtype = rt.act_dtype
 
     def forward(self, h, ctx, cache, residual, writes: bool = True) -> None:
-        y = linear(h, self.w_y, out_dtype=self.act_dtype)
-        x = linear(h, self.w_x, out_dtype=self.act_dtype)
+        yx = linear(h, self.w_yx, out_dtype=self.act_dtype)
+        y, x = yx[:, :self.width], yx[:, self.width:]
         u = ops.causal_conv(x, self.conv_w, cache.tail if self.conv_taps > 1 else None, ctx, in_bias=self.x_b,
                             out_bias=self.conv_b)
         out = ops.rglru(u, y, self.w_gates, self.ra_b, self.ri_b, self.lam, self.y_b, cache.state, ctx)
