@@ -666,6 +666,16 @@ def gemm_swiglu(a: torch.Tensor, w_gate_up, interleaved: bool = False) -> torch.
     return swiglu(gu, interleaved)
 
 
+class Fresh:
+    """Stands for a float32 [rows, n] sum that does not exist yet, where a part expects the stream it adds to: the first
+    product "added" to it is simply stored, and the result is found in ``tensor`` (parts.linear.linear).  A block that
+    norms a sublayer's output before adding it to the stream hands this to parts that add through one last product, and
+    saves clearing a buffer and reading it back."""
+
+    def __init__(self):
+        self.tensor: Optional[torch.Tensor] = None
+
+
 class Prenormed:
     """What a product that added into the residual stream left for the RMSNorm after it
     (gemm_accumulate_emit): ``xb`` = bfloat16(residual * g) [m, width] and ``parts`` [blocks, m], block

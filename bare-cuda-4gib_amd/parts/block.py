@@ -83,15 +83,25 @@ class SandwichBlock(Part):
         if self.mixer_conv is not None:
             h = self.mixer_conv.forward(h, ctx, cache.conv, add_input=True)
             mixer_cache = cache.mixer
-        y = torch.zeros_like(x)
+        y = self._sum_for(self.mixer, x)
         self.mixer.forward(h, ctx, mixer_cache, y, writes)
-        self.mixer_post_norm.add_to(x, y)
+        self.mixer_post_norm.add_to(x, self._sum_of(y))
         if self.ffn is not None:
-            y = torch.zeros_like(x)
+            y = self._sum_for(self.ffn, x)
             # (a feed-forward that says so gets the norm not yet computed: its first product absorbs it for few rows)
             lazy = getattr(self.ffn, "accepts_lazy_norm", False)
             self.ffn.forward(Normed(x, self.ffn_norm, ctx) if lazy else self.ffn_norm.forward(x, ctx), ctx, y)
-            self.ffn_post_norm.add_to(x, y)
+            self.ffn_post_norm.add_to(x, self._sum_of(y))
+
+    @staticmethod
+    def _sum_for(part, x):
+        """What the part adds its output to: nothing yet (ops.Fresh) for a part that says its output is one last product
+        through parts.linear.linear (``adds_one_product``), else a cleared buffer."""
+        return ops.Fresh() if getattr(part, "adds_one_product", False) else torch.zeros_like(x)
+
+    @staticmethod
+    def _sum_of(y):
+        return y.tensor if isinstance(y, ops.Fresh) else y
 
 
 register_part("block", "prenorm", PreNormBlock)

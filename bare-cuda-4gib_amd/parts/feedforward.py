@@ -60,6 +60,7 @@ class DenseXIELU(Part):
     category = "feedforward"
     graph_safe = True     # launches kernels only: may run inside a captured graph
     accepts_lazy_norm = True
+    adds_one_product = True   # the output is one last product through linear(): a block may hand it ops.Fresh
 
     def __init__(self, hidden_size: int, intermediate_size: int):
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)

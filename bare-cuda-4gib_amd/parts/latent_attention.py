@@ -25,6 +25,7 @@ class LatentAttention(Part):
     latents, so no key or value is ever made per head and token; scores, weights and the sums are float32."""
     category = "mixer"
     graph_safe = True     # launches kernels only: may run inside a captured graph
+    adds_one_product = True   # the output is one last product through linear(): a block may hand it ops.Fresh
 
     def __init__(self, hidden_size: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, scale: float,
                  rot_dims: int, rot_base: float, eps: float, sink: bool = True, window: int = 0):

@@ -39,6 +39,11 @@ def linear(x: Union[torch.Tensor, Normed], w, out_dtype: Optional[torch.dtype] =
     itself (ops.Finished) where the product cuts k over workgroups anyway -- the kernel that adds the parts
     up norms the stream on its way, which serves every reader -- or else, if the reader takes that, the parts
     of the norm that a product can finish (ops.Prenormed)."""
+    if isinstance(accumulate_into, ops.Fresh):        # nothing to add to yet: the product itself, in float32
+        if accumulate_into.tensor is not None:
+            return linear(x, w, accumulate_into=accumulate_into.tensor, ctx=ctx)
+        accumulate_into.tensor = linear(x, w, out_dtype=torch.float32)
+        return accumulate_into.tensor
     if isinstance(x, Normed):
         if accumulate_into is None and out_dtype in (torch.bfloat16, torch.float32):
             epi = ops.EPI_STORE_BF16 if out_dtype == torch.bfloat16 else ops.EPI_STORE_F32

@@ -21,6 +21,7 @@ class RGLRU(Part):
     the convolution's last taps - 1 inputs."""
     category = "mixer"
     graph_safe = True     # launches kernels only: may run inside a captured graph
+    adds_one_product = True   # the output is one last product through linear(): a block may hand it ops.Fresh
 
     def __init__(self, hidden_size: int, width: int, blocks: int, conv_taps: int):
         if hidden_size <= 0 or width <= 0 or blocks <= 0 or width % blocks or conv_taps < 1:
