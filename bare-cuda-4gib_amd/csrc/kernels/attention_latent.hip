@@ -57,6 +57,23 @@ __global__ __launch_bounds__(kPrepBlock) void latent_prepare_kernel(
   extern __shared__ float cs[];                     // [dims / 2][2]: the row's cosines and sines
   const long row = blockIdx.x;
   for (int i = threadIdx.x; i < dims; i += kPrepBlock) cs[i] = angles[row * dims + i];
+  // (two workgroups a row: one norms and stores the cache row, the other rotates the queries)
+  if (blockIdx.y == 1) {
+    __syncthreads();
+    const T* qr = q + row * q_row;
+    float* ql = q_lat + row * heads * (rank + rot);
+    for (int e = threadIdx.x; e < heads * rot; e += kPrepBlock) {
+      const int h = e / rot, i = e % rot;
+      const T* part = qr + h * (plain + rot) + plain;
+      float v = to_float(part[i]);
+      if (i < dims) {
+        const float c = cs[2 * (i / 2)], s = cs[2 * (i / 2) + 1], other = to_float(part[i ^ 1]);
+        v = (i & 1) ? v * c + other * s : v * c - other * s;
+      }
+      ql[h * (rank + rot) + rank + i] = v;
+    }
+    return;
+  }
   const T* lat = dkv + row * dkv_row;
   float ss = 0.f;
   for (int i = threadIdx.x; i < rank; i += kPrepBlock) {
@@ -75,18 +92,6 @@ __global__ __launch_bounds__(kPrepBlock) void latent_prepare_kernel(
       }
       to[rank + i] = from_float<T>(v);
     }
-  }
-  const T* qr = q + row * q_row;
-  float* ql = q_lat + row * heads * (rank + rot);
-  for (int e = threadIdx.x; e < heads * rot; e += kPrepBlock) {
-    const int h = e / rot, i = e % rot;
-    const T* part = qr + h * (plain + rot) + plain;
-    float v = to_float(part[i]);
-    if (i < dims) {
-      const float c = cs[2 * (i / 2)], s = cs[2 * (i / 2) + 1], other = to_float(part[i ^ 1]);
-      v = (i & 1) ? v * c + other * s : v * c - other * s;
-    }
-    ql[h * (rank + rot) + rank + i] = v;
   }
 }
 
@@ -326,11 +331,11 @@ extern "C" int bc4g_latent_prepare(const void* q, const void* dkv, int dtype, co
   hipStream_t s = static_cast<hipStream_t>(stream);
   const size_t lds = static_cast<size_t>(dims > 0 ? dims : 2) * sizeof(float);
   if (dtype == kF32)
-    latent_prepare_kernel<float><<<n_rows, kPrepBlock, lds, s>>>(static_cast<const float*>(q), static_cast<const float*>(dkv), g,
+    latent_prepare_kernel<float><<<dim3(n_rows, 2), kPrepBlock, lds, s>>>(static_cast<const float*>(q), static_cast<const float*>(dkv), g,
                                                                  eps, angles, slot_map, static_cast<float*>(cache), q_lat,
                                                                  heads, plain, rot, rank, dims, q_row, dkv_row);
   else if (dtype == kBF16)
-    latent_prepare_kernel<bf16_t><<<n_rows, kPrepBlock, lds, s>>>(static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(dkv),
+    latent_prepare_kernel<bf16_t><<<dim3(n_rows, 2), kPrepBlock, lds, s>>>(static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(dkv),
                                                                   g, eps, angles, slot_map, static_cast<bf16_t*>(cache),
                                                                   q_lat, heads, plain, rot, rank, dims, q_row, dkv_row);
   else return fail("latent_prepare: unknown dtype %d", dtype);

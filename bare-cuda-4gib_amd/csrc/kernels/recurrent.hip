@@ -31,9 +31,9 @@ __device__ inline float conv_input(const T* in, const float* in_bias, long at, i
 template <typename T>
 __global__ void causal_conv_kernel(const T* __restrict__ in, const float* __restrict__ in_bias,
                                    const float* __restrict__ w, const float* __restrict__ out_bias, int add_input,
-                                   T* __restrict__ out, const T* __restrict__ state, const int32_t* __restrict__ row_seq,
+                                   T* __restrict__ out, T* state, const int32_t* __restrict__ row_seq,
                                    const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slots,
-                                   long total, int channels, int taps, long in_row) {
+                                   long total, int channels, int taps, long in_row, int single_rows) {
   const long stride = static_cast<long>(blockDim.x) * gridDim.x;
   for (long idx = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; idx < total; idx += stride) {
     const int c = static_cast<int>(idx % channels);
@@ -41,7 +41,7 @@ __global__ void causal_conv_kernel(const T* __restrict__ in, const float* __rest
     const int s = row_seq[t];
     const long start = seq_start[s];
     const int local = static_cast<int>(t - start);
-    const T* tail = state + static_cast<long>(seq_slots[s]) * (taps - 1) * channels;
+    T* tail = state + static_cast<long>(seq_slots[s]) * (taps - 1) * channels;
     float acc = out_bias ? out_bias[c] : 0.f;
     for (int j = 0; j < taps; ++j) {
       const int src = local - (taps - 1) + j;
@@ -51,6 +51,10 @@ __global__ void causal_conv_kernel(const T* __restrict__ in, const float* __rest
     }
     if (add_input) acc += to_float(in[t * in_row + c]);
     out[idx] = from_float<T>(acc);
+    if (single_rows) {      // every request brings one row: this thread alone touches the tail of (request, channel)
+      for (int i = 0; i + 1 < taps - 1; ++i) tail[static_cast<long>(i) * channels + c] = tail[static_cast<long>(i + 1) * channels + c];
+      if (taps > 1) tail[static_cast<long>(taps - 2) * channels + c] = from_float<T>(conv_input(in, in_bias, t, c, in_row));
+    }
   }
 }
 
@@ -64,9 +68,10 @@ __device__ inline void widen8(const uint4 v, float (&f)[8]) {
 
 __global__ void causal_conv_pieces_kernel(const bf16_t* __restrict__ in, const float* __restrict__ in_bias,
                                           const float* __restrict__ w, const float* __restrict__ out_bias, int add_input,
-                                          bf16_t* __restrict__ out, const bf16_t* __restrict__ state,
+                                          bf16_t* __restrict__ out, bf16_t* state,
                                           const int32_t* __restrict__ row_seq, const int32_t* __restrict__ seq_start,
-                                          const int32_t* __restrict__ seq_slots, long total, int channels, int taps, long in_row) {
+                                          const int32_t* __restrict__ seq_slots, long total, int channels, int taps, long in_row,
+                                          int single_rows) {
   const int pieces = channels / 8;
   const long stride = static_cast<long>(blockDim.x) * gridDim.x;
   for (long idx = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; idx < total; idx += stride) {
@@ -75,7 +80,7 @@ __global__ void causal_conv_pieces_kernel(const bf16_t* __restrict__ in, const f
     const int s = row_seq[t];
     const long start = seq_start[s];
     const int local = static_cast<int>(t - start);
-    const bf16_t* tail = state + static_cast<long>(seq_slots[s]) * (taps - 1) * channels;
+    bf16_t* tail = state + static_cast<long>(seq_slots[s]) * (taps - 1) * channels;
     float acc[8], bias[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = out_bias ? out_bias[c0 + e] : 0.f, bias[e] = in_bias ? in_bias[c0 + e] : 0.f;
@@ -108,6 +113,20 @@ __global__ void causal_conv_pieces_kernel(const bf16_t* __restrict__ in, const f
     for (int e = 0; e < 4; ++e)
       o[e] = static_cast<unsigned>(bf16_bits_from_float(acc[2 * e])) | (static_cast<unsigned>(bf16_bits_from_float(acc[2 * e + 1])) << 16);
     *reinterpret_cast<uint4*>(out + t * channels + c0) = make_uint4(o[0], o[1], o[2], o[3]);
+    if (single_rows) {      // every request brings one row: this thread alone touches the tail of (request, these channels)
+      for (int i = 0; i + 1 < taps - 1; ++i)
+        *reinterpret_cast<uint4*>(tail + static_cast<long>(i) * channels + c0) = load16(tail + static_cast<long>(i + 1) * channels + c0);
+      if (taps > 1) {
+        float v[8];
+        widen8(load16(in + t * in_row + c0), v);
+        unsigned k[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          k[e] = static_cast<unsigned>(bf16_bits_from_float(v[2 * e] + bias[2 * e])) |
+                 (static_cast<unsigned>(bf16_bits_from_float(v[2 * e + 1] + bias[2 * e + 1])) << 16);
+        *reinterpret_cast<uint4*>(tail + static_cast<long>(taps - 2) * channels + c0) = make_uint4(k[0], k[1], k[2], k[3]);
+      }
+    }
   }
 }
 
@@ -211,12 +230,15 @@ extern "C" int bc4g_causal_conv(const void* in, int dtype, const float* in_bias,
   if (n_rows == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const long total = static_cast<long>(n_rows) * channels, per_seq = static_cast<long>(n_seqs) * channels;
+  // every request brings one row (a decode step): the thread that computes a row's channel also moves its tail
+  const int single_rows = n_rows == n_seqs ? 1 : 0;
 #define BC4G_CONV(T)                                                                                                      \
   do {                                                                                                                    \
     causal_conv_kernel<T><<<grid_for(total), kBlock, 0, s>>>(static_cast<const T*>(in), in_bias, w, out_bias, add_input, \
-                                                             static_cast<T*>(out), static_cast<const T*>(state), row_seq, \
-                                                             seq_start, seq_slots, total, channels, taps, in_row);        \
-    if (taps > 1)                                                                                                         \
+                                                             static_cast<T*>(out), static_cast<T*>(state), row_seq,       \
+                                                             seq_start, seq_slots, total, channels, taps, in_row,         \
+                                                             single_rows);                                                \
+    if (taps > 1 && !single_rows)                                                                                         \
       causal_conv_state_kernel<T><<<grid_for(per_seq), kBlock, 0, s>>>(static_cast<const T*>(in), in_bias,                \
                                                                        static_cast<T*>(state), seq_start, seq_slots,      \
                                                                        per_seq, channels, taps, in_row);                  \
@@ -227,9 +249,9 @@ extern "C" int bc4g_causal_conv(const void* in, int dtype, const float* in_bias,
   if (dtype == kF32) BC4G_CONV(float);
   else if (pieces) {
     causal_conv_pieces_kernel<<<grid_for(total / 8), kBlock, 0, s>>>(
-        static_cast<const bf16_t*>(in), in_bias, w, out_bias, add_input, static_cast<bf16_t*>(out), static_cast<const bf16_t*>(state),
-        row_seq, seq_start, seq_slots, total / 8, channels, taps, in_row);
-    if (taps > 1)
+        static_cast<const bf16_t*>(in), in_bias, w, out_bias, add_input, static_cast<bf16_t*>(out), static_cast<bf16_t*>(state),
+        row_seq, seq_start, seq_slots, total / 8, channels, taps, in_row, single_rows);
+    if (taps > 1 && !single_rows)
       causal_conv_state_kernel<bf16_t><<<grid_for(per_seq), kBlock, 0, s>>>(static_cast<const bf16_t*>(in), in_bias,
                                                                             static_cast<bf16_t*>(state), seq_start, seq_slots,
                                                                             per_seq, channels, taps, in_row);
