@@ -362,6 +362,43 @@ def test_latent_attention_finds_one_key_among_hundreds(dtype, needle, sizes):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("sizes", [(3, 20, 12), (4, 48, 16), (16, 128, 32)])
+@pytest.mark.parametrize("back", [49, 50])
+def test_latent_attention_within_a_window(dtype, sizes, back):
+    """The part takes a window as a parameter (this design sets none): with a window of 50 a row sees the 50 keys up to
+    its own.  A key made to stand out 49 places back takes the weight, the same key 50 places back is not seen at all --
+    as a decoded token and in a portion whose rows' windows begin at different keys."""
+    from bare_cuda_4gib_amd.csrc import ops
+    torch.manual_seed(back)
+    (H, rank, rot), dev, n, P, scale, window = sizes, "cuda:0", 130, 16, 0.3, 50
+    rows = (torch.randn(n, rank + rot) * 0.3).to(dtype)
+    q = torch.randn(H, rank + rot)
+    needle = n - 1 - back
+    rows[needle] = (q[0] / float(q[0] @ q[0]) * 14.0 / scale).to(dtype)
+    pages = torch.randperm(20)[:-(-n // P)]
+    cache = torch.full((21, P, rank + rot), float("nan"), dtype=dtype, device=dev)
+    for j in range(n):
+        cache[pages[j // P], j % P] = rows[j].to(dev)
+    table = pages.to(torch.int32).view(1, -1).to(dev)
+    tensor_cores = dtype == torch.bfloat16 and ops.attention_latent_mfma_takes(cache, rank, rot)
+    tol = 3e-2 if tensor_cores else 2e-5
+    for lengths, cached in (([1], [n - 1]), ([5], [n - 5])):
+        ctx = step_context(lengths, cached, [0])
+        q_lat = q.view(1, H, -1).repeat(lengths[0], 1, 1).contiguous().to(dev)
+        got = ops.attention_latent(q_lat, cache, None, table, ctx, H, rank, rot, P, window, scale).cpu().double()
+        for k in range(lengths[0]):
+            pos = cached[0] + k
+            lo = max(0, pos - window + 1)
+            for a in range(H):
+                s = (rows[lo:pos + 1].double() @ q[a].double()) * scale
+                w = torch.softmax(s, 0)                       # (no sink here)
+                want = w @ rows[lo:pos + 1, :rank].double()
+                assert torch.allclose(got[k, a], want, atol=tol * float(want.abs().max()), rtol=tol), (back, pos, a)
+                if a == 0 and lo <= needle:
+                    assert float(w[needle - lo]) > 0.9
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_latent_rows_are_normed_rotated_and_written_to_their_slots(dtype):
     from bare_cuda_4gib_amd.csrc import ops
     torch.manual_seed(4)
