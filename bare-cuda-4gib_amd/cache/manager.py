@@ -116,22 +116,24 @@ def bytes_per_page(specs: Iterable[Any], page_tokens: int, dtype: torch.dtype) -
 
 
 def _retention(spec):
-    """(group key, first_kept, keeps everything) of a per-token spec: its own statement, or what its
-    ``window`` says (0 or absent: every token is kept)."""
+    """(group key, first_kept, keeps everything, leading tokens always kept) of a per-token spec: its own statement,
+    or what its ``window`` says (0 or absent: every token is kept)."""
     window = int(getattr(spec, "window", 0))
+    always = int(spec.always_kept()) if hasattr(spec, "always_kept") else 0
     if hasattr(spec, "first_kept"):
         key = spec.group_key() if hasattr(spec, "group_key") else ("rule", type(spec).__name__, window)
-        return key, spec.first_kept, key == ("window", 0)
+        return key, spec.first_kept, key == ("window", 0), always
     if window > 0:
-        return ("window", window), (lambda length: max(0, length - window + 1)), False
-    return ("window", 0), (lambda length: 0), True
+        return ("window", window), (lambda length: max(0, length - window + 1)), False, always
+    return ("window", 0), (lambda length: 0), True, 0
 
 
 class _Group:
-    def __init__(self, window: int, num_pages: int, first_kept, keeps_all: bool):
+    def __init__(self, window: int, num_pages: int, first_kept, keeps_all: bool, always_kept: int = 0):
         self.window = window                 # (what the views show; the rule itself is first_kept)
         self.first_kept = first_kept         # length -> earliest token still read by a query at `length` or later
         self.keeps_all = keeps_all
+        self.always_kept = always_kept       # leading tokens that are read whatever first_kept says
         self.pool = PagePool(num_pages)
         self.streams: List[Hashable] = []
 
@@ -194,10 +196,10 @@ class CacheManager:
             return BundleView(made)
         if getattr(spec, "per_token", None) is True and hasattr(spec, "page_tensors"):
             window = int(getattr(spec, "window", 0))
-            key, first_kept, keeps_all = _retention(spec)
+            key, first_kept, keeps_all, always = _retention(spec)
             group = self.groups.get(key)
             if group is None:
-                group = self.groups[key] = _Group(window, num_pages, first_kept, keeps_all)
+                group = self.groups[key] = _Group(window, num_pages, first_kept, keeps_all, always)
             group.streams.append(sid)
             tensors = {}
             for name, entry in spec.page_tensors(page_tokens).items():
@@ -340,6 +342,8 @@ class CacheManager:
                 continue
             # the next query sits at position r.length; pages wholly before what it and later ones read go back
             first_needed = max(0, int(group.first_kept(r.length))) // self.page_tokens
+            # (the pages of the leading tokens that every query reads stay: the walk begins behind them)
+            r.released[g] = max(r.released[g], min(self.pages_for(group.always_kept), len(t)))
             for idx in range(r.released[g], min(first_needed, len(t))):
                 self._give_back(g, t[idx])
                 t[idx] = -1
@@ -396,7 +400,8 @@ class CacheManager:
             most = 0
             for p in range(0, max(total_tokens, 1)):
                 upto = min(p + max(portion, 1), total_tokens)
-                most = max(most, -(-upto // P) - max(0, int(group.first_kept(p))) // P)
+                passed = max(0, int(group.first_kept(p))) // P
+                most = max(most, -(-upto // P) - passed + min(self.pages_for(group.always_kept), passed))
             out[g] = most
         if len(self._peaks) > 4096:
             self._peaks.clear()

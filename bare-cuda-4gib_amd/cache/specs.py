@@ -11,7 +11,8 @@ per token   ``per_token = True``.  ``page_tensors(page_tokens)`` names the tenso
             wholly before it go back to their pool; ``group_key()`` names the rule -- specs with equal
             keys share a page pool and one block table per request.  A spec that has neither is read
             by its ``window`` (0 or absent = keep everything; W = a query reads the W tokens up to and
-            including its own).
+            including its own).  ``always_kept()`` (optional) is the number of leading tokens that stay
+            whatever ``first_kept`` says: the pages that hold them are never given back before the request ends.
 per request ``per_token = False``.  ``slot_tensors()`` names the tensors of ONE request slot
             (name -> (shape, dtype name)); the manager allocates ``[max_requests, *shape]`` of each and
             zeroes a slot when a request is admitted to it.
@@ -84,6 +85,36 @@ class PagedLatent:
 
     def first_kept(self, length: int) -> int:
         return max(0, length - self.window + 1) if self.window > 0 else 0
+
+
+@dataclasses.dataclass(frozen=True)
+class PagedHeads:
+    """Keys and values per token, in pages, with head counts and sizes of their own: keys
+    ``[page, key_heads, token, key_dim]``, values ``[page, value_heads, token, value_dim]`` (a token's elements side by
+    side in both).  ``window`` 0 keeps every token; otherwise a query reads the last ``window`` tokens and, whatever its
+    position, the first ``keep_first`` tokens of the sequence: pages between those and the window are given back."""
+    key_heads: int
+    key_dim: int
+    value_heads: int
+    value_dim: int
+    window: int = 0
+    keep_first: int = 0
+    per_token = True
+
+    def page_tensors(self, page_tokens: int) -> Dict[str, Tuple[int, ...]]:
+        return {"k": (self.key_heads, page_tokens, self.key_dim), "v": (self.value_heads, page_tokens, self.value_dim)}
+
+    def group_key(self):
+        if self.window <= 0 or self.keep_first <= 0:
+            return ("window", max(self.window, 0))
+        return ("window", self.window, "first", self.keep_first)
+
+    def first_kept(self, length: int) -> int:
+        return max(0, length - self.window + 1) if self.window > 0 else 0
+
+    def always_kept(self) -> int:
+        """The leading tokens that every later query reads, wherever the window stands."""
+        return self.keep_first if self.window > 0 else 0
 
 
 @dataclasses.dataclass(frozen=True)

@@ -280,3 +280,55 @@ int bc4g_attention_latent_mfma(const float* q_lat, float* out, float* part_o, fl
                                const int32_t* seq_ctx, int n_seqs, int n_tokens, int most_tokens, int heads, int rank, int rot,
                                int page_tokens, int window, float scale, int n_splits, void* stream);
 }
+
+extern "C" {
+// out[t, i] = g sigmoid(slope g) (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit); gu [T, 2 I] holds a row's gates,
+// then its ups.
+int bc4g_clamped_glu(const void* gu, void* out, int dtype, float limit, float slope, int n_rows, int inter, void* stream);
+
+// A residual stream in n copies, x [T, n, H] float32 (streams.hip).  read: out[r] = N(sum_s read[s] x[rows ? rows[r] : r, s])
+// with N(u) = (tanh(alpha u) g + b) out_scale (alpha null: out = the sum; read null: every copy counts once).  write:
+// x'[t] = sum_s mix[s, t] x[s] + write[t] y for all copies at once, and with next_out also the next reader's input
+// N(sum_t next_read[t] x'[t]).  fill: every copy = in.  At most 8 copies.
+int bc4g_streams_read(const float* x, const int32_t* rows, const float* read, const float* alpha, const float* g, const float* b,
+                      float out_scale, void* out, int out_dtype, int n_rows, int n_streams, int hidden, void* stream);
+int bc4g_streams_write(float* x, const float* y, const float* mix, const float* write, const float* next_read,
+                       const float* alpha, const float* g, const float* b, void* next_out, int out_dtype, int n_rows,
+                       int n_streams, int hidden, void* stream);
+int bc4g_streams_fill(const float* in, float* out, int n_rows, int n_streams, int hidden, void* stream);
+
+// table [T, half, 2]: cos and sin of positions[t] * freqs[i], times amp; the angle in double (decay_scan.hip).
+int bc4g_rotary_table(const int32_t* positions, const double* freqs, double amp, float* table, int n_rows, int half, void* stream);
+// Per (row, head) of in [T, heads, dim] (rows in_row apart): + bias [heads, dim], RMS norm over dim with weight norm_w [dim]
+// (null: none), rotation of the first 2 * half elements by the table (element i with element i + half), times factor;
+// into out [T, heads, dim] (rows out_row apart) or, with slot_map (slot = page * page_tokens + offset), into a cache
+// at out + page * page_stride + head * head_stride + offset * token_stride.  dim at most 256.
+int bc4g_heads_prepare(const void* in, int in_dtype, long in_row, const float* bias, const float* norm_w, float eps,
+                       const float* table, int half, float factor, void* out, int out_dtype, long out_row,
+                       const int32_t* slot_map, int page_tokens, long page_stride, long head_stride, long token_stride,
+                       int n_rows, int heads, int dim, void* stream);
+// out[t, h] = o[t, h] / sqrt(mean(o[t, h]^2) + eps) (* w [vdim]) * factor * act(gate[t, h]); act 0: none, 1: silu,
+// 2: sigmoid; o float32 [T, heads, vdim]; vdim at most 256.
+int bc4g_heads_finish(const float* o, const float* w, float eps, float factor, const void* gate, int gate_dtype, long gate_row,
+                      int act, void* out, int out_dtype, int n_rows, int heads, int vdim, void* stream);
+// S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T (q_t q_scale) along every request's rows, from state
+// [slots, heads, dim, vdim] (float32) and back into it; out float32 [T, heads, vdim].  a_t = head_decay[head], or with
+// gate logits z [T, heads, dim]: sigmoid(z + z_bias)^inv_tau.  Requests that bring more than 64 rows are walked in
+// chunks: chunk_state [chunks, heads, dim, vdim], chunk_decay [chunks, heads, dim] (float32 scratch) and chunk_base [S],
+// the first chunk of every request among all chunks of requests that have two or more.  dim at most 256.
+int bc4g_decay_scan(const void* q, int q_dtype, long q_row, float q_scale, const void* k, int k_dtype, long k_row,
+                    const void* v, int v_dtype, long v_row, const float* head_decay, const void* z, int z_dtype, long z_row,
+                    const float* z_bias, float inv_tau, float* out, float* state, float* chunk_state, float* chunk_decay,
+                    const int32_t* seq_start, const int32_t* seq_slots, const int32_t* chunk_base, int n_rows, int n_seqs,
+                    int most_rows, int heads, int dim, int vdim, void* stream);
+
+// Attention with one or two score maps per query head over the same values (attention_maps.hip): q float32
+// [T, heads, maps, dim]; keys [page, kv_head * maps + map, token, dim], values [page, kv_head, token, vdim]; a row at p
+// sees j <= p with p - j < window or j < keep_first (window 0: all).  o = a1 - lambda a2 (one map: a1), with normalize
+// divided by sqrt(mean(o^2) + eps), times factor, times act(gate) (1: silu, 2: sigmoid; gate null: none).
+int bc4g_attention_maps(const float* q, long q_row, const void* k_cache, const void* v_cache, int cache_dtype,
+                        const int32_t* block_table, int table_stride, const int32_t* row_seq, const int32_t* positions,
+                        float lambda, int normalize, float eps, float factor, const void* gate, int gate_dtype, long gate_row,
+                        int gate_act, void* out, int out_dtype, int n_rows, int n_heads, int n_kv_heads, int maps, int dim,
+                        int vdim, int page_tokens, int window, int keep_first, float scale, void* stream);
+}

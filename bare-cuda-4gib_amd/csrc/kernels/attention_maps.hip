@@ -1,0 +1,177 @@
+// Softmax attention over a paged cache whose query heads carry one or two score maps over the same values
+// (differential attention: o = a1 - lambda a2), with a window of the last keys plus the first few keys of the
+// sequence, keys and values of different sizes, and the head's output optionally divided by its root mean square,
+// scaled and gated.  Plain float arithmetic on float or bfloat16 caches: scores, weights and sums are float32.
+//
+// A row at position p sees key j if j <= p and (window == 0 or p - j < window or j < keep_first); kept keys keep their
+// own positions (they were rotated when they were written).  One wave per (row, query head): the visible keys are
+// walked in tiles of 64 in ascending order -- the kept first keys, then the window -- with a running maximum and sum per
+// map (lane = key for the scores, lane = value dimension for the sums, a tile's values read once for both maps).
+// Pages that hold no visible key are never touched.
+//
+// Caches: keys [page, kv_head * maps + map, token, dim], values [page, kv_head, token, vdim].
+#include <float.h>
+#include <math.h>
+
+#include "api.h"
+#include "common.h"
+
+namespace bc4g {
+namespace {
+
+constexpr int kMaxDim = 256;     // of a map's queries and keys
+constexpr int kMaxVdim = 256;    // of a head's values
+constexpr int kPerLane = kMaxVdim / kWave;
+
+__device__ inline float4 load_four(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ inline float4 load_four(const bf16_t* p) {
+  const uint2 bits = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(bits.x << 16), __uint_as_float(bits.x & 0xffff0000u),
+                     __uint_as_float(bits.y << 16), __uint_as_float(bits.y & 0xffff0000u));
+}
+
+__device__ inline float gate_of(const void* gate, int dtype, long idx, int act) {
+  const float z = dtype == kF32 ? static_cast<const float*>(gate)[idx] : to_float(static_cast<const bf16_t*>(gate)[idx]);
+  return act == 1 ? z / (1.0f + expf(-z)) : 1.0f / (1.0f + expf(-z));
+}
+
+template <typename T, int MAPS>
+__global__ __launch_bounds__(kWave) void attention_maps_kernel(
+    const float* __restrict__ q, long q_row, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seq,
+    const int32_t* __restrict__ positions, float lambda, int normalize, float eps, float factor,
+    const void* __restrict__ gate, int gate_dtype, long gate_row, int gate_act, void* __restrict__ out, int out_dtype,
+    int n_heads, int n_kv_heads, int dim, int vdim, int page_tokens, int window, int keep_first, float scale) {
+  __shared__ float q_s[MAPS][kMaxDim];
+  __shared__ float p_s[MAPS][kWave];
+  const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const int kvh = head / (n_heads / n_kv_heads);
+  const int pos = positions[row];
+  const int32_t* table = block_table + static_cast<long>(row_seq[row]) * table_stride;
+  for (int m = 0; m < MAPS; ++m)
+    for (int c = lane; c < dim; c += kWave) q_s[m][c] = q[row * q_row + (static_cast<long>(head) * MAPS + m) * dim + c];
+  __syncthreads();
+
+  const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int kept = window > 0 ? (keep_first < first ? keep_first : first) : 0;      // kept keys before the window
+  const int total = kept + (pos - first + 1);
+  const bool by_four = dim % 4 == 0 && reinterpret_cast<uintptr_t>(k_cache) % (4 * sizeof(T)) == 0;
+  float mx[MAPS], sum[MAPS], acc[MAPS][kPerLane];
+#pragma unroll
+  for (int m = 0; m < MAPS; ++m) {
+    mx[m] = -INFINITY, sum[m] = 0.f;
+#pragma unroll
+    for (int i = 0; i < kPerLane; ++i) acc[m][i] = 0.f;
+  }
+  for (int v0 = 0; v0 < total; v0 += kWave) {
+    const int vi = v0 + lane;
+    const bool seen = vi < total;
+    const int j = vi < kept ? vi : first + (vi - kept);
+    const long page = seen ? table[j / page_tokens] : 0;
+    const int off = j % page_tokens;
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+      float dot = 0.f;
+      if (seen) {
+        const T* kp = k_cache + ((page * (n_kv_heads * MAPS) + kvh * MAPS + m) * page_tokens + off) * dim;
+        if (by_four) {
+          for (int c = 0; c < dim; c += 4) {
+            const float4 kk = load_four(kp + c);
+            dot = fmaf(q_s[m][c], kk.x, dot), dot = fmaf(q_s[m][c + 1], kk.y, dot);
+            dot = fmaf(q_s[m][c + 2], kk.z, dot), dot = fmaf(q_s[m][c + 3], kk.w, dot);
+          }
+        } else {
+          for (int c = 0; c < dim; ++c) dot = fmaf(q_s[m][c], to_float(kp[c]), dot);
+        }
+      }
+      const float sc = seen ? dot * scale : -INFINITY;
+      const float m_new = fmaxf(mx[m], wave_max(sc));       // finite: the tile's first key is visible
+      const float p = seen ? expf(sc - m_new) : 0.f;
+      const float alpha = expf(mx[m] - m_new);               // 0 on the first tile
+      sum[m] = sum[m] * alpha + wave_sum(p);
+      mx[m] = m_new;
+      p_s[m][lane] = p;
+#pragma unroll
+      for (int i = 0; i < kPerLane; ++i) acc[m][i] *= alpha;
+    }
+    __syncthreads();
+    const int n_here = total - v0 < kWave ? total - v0 : kWave;
+    for (int jj = 0; jj < n_here; ++jj) {
+      const int vj = v0 + jj;
+      const int jk = vj < kept ? vj : first + (vj - kept);
+      const long pg = table[jk / page_tokens];
+      const T* vrow = v_cache + ((pg * n_kv_heads + kvh) * page_tokens + jk % page_tokens) * vdim;
+#pragma unroll
+      for (int i = 0; i < kPerLane; ++i) {
+        const int c = lane + i * kWave;
+        if (c < vdim) {
+          const float vv = to_float(vrow[c]);
+#pragma unroll
+          for (int m = 0; m < MAPS; ++m) acc[m][i] = fmaf(p_s[m][jj], vv, acc[m][i]);
+        }
+      }
+    }
+    __syncthreads();
+  }
+  float o[kPerLane];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < kPerLane; ++i) {
+    o[i] = acc[0][i] / sum[0];
+    if (MAPS == 2) o[i] -= lambda * (acc[MAPS - 1][i] / sum[MAPS - 1]);
+    ss = fmaf(o[i], o[i], ss);          // (lanes beyond vdim hold zeros)
+  }
+  const float mult = normalize ? factor / sqrtf(wave_sum(ss) / static_cast<float>(vdim) + eps) : factor;
+#pragma unroll
+  for (int i = 0; i < kPerLane; ++i) {
+    const int c = lane + i * kWave;
+    if (c >= vdim) break;
+    float r = o[i] * mult;
+    if (gate) r *= gate_of(gate, gate_dtype, row * gate_row + static_cast<long>(head) * vdim + c, gate_act);
+    const long at = (static_cast<long>(row) * n_heads + head) * vdim + c;
+    if (out_dtype == kF32) static_cast<float*>(out)[at] = r;
+    else static_cast<bf16_t*>(out)[at] = from_float<bf16_t>(r);
+  }
+}
+
+}  // namespace
+}  // namespace bc4g
+
+using namespace bc4g;
+
+extern "C" int bc4g_attention_maps(const float* q, long q_row, const void* k_cache, const void* v_cache, int cache_dtype,
+                                   const int32_t* block_table, int table_stride, const int32_t* row_seq,
+                                   const int32_t* positions, float lambda, int normalize, float eps, float factor,
+                                   const void* gate, int gate_dtype, long gate_row, int gate_act, void* out, int out_dtype,
+                                   int n_rows, int n_heads, int n_kv_heads, int maps, int dim, int vdim, int page_tokens,
+                                   int window, int keep_first, float scale, void* stream) {
+  BC4G_REQUIRE(n_rows >= 0 && n_heads > 0 && n_heads <= 65535 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
+               "attention_maps: bad sizes T=%d heads=%d/%d", n_rows, n_heads, n_kv_heads);
+  BC4G_REQUIRE((maps == 1 || maps == 2) && dim > 0 && dim <= kMaxDim && vdim > 0 && vdim <= kMaxVdim,
+               "attention_maps: maps=%d (1 or 2), dim=%d (at most %d), vdim=%d (at most %d)", maps, dim, kMaxDim, vdim, kMaxVdim);
+  BC4G_REQUIRE(page_tokens > 0 && table_stride > 0 && window >= 0 && keep_first >= 0,
+               "attention_maps: bad cache sizes page_tokens=%d table_stride=%d window=%d keep_first=%d", page_tokens,
+               table_stride, window, keep_first);
+  BC4G_REQUIRE(q && k_cache && v_cache && block_table && row_seq && positions && out &&
+               q_row >= static_cast<long>(n_heads) * maps * dim && (!gate || gate_row >= static_cast<long>(n_heads) * vdim) &&
+               (gate_act == 1 || gate_act == 2 || !gate) && (out_dtype == kF32 || out_dtype == kBF16) &&
+               (!gate || gate_dtype == kF32 || gate_dtype == kBF16),
+               "attention_maps: a tensor is missing, a row is shorter than its heads, or a dtype is unknown");
+  if (n_rows == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid(n_rows, n_heads);
+#define BC4G_MAPS(T, M)                                                                                                   \
+  attention_maps_kernel<T, M><<<grid, kWave, 0, s>>>(q, q_row, static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), \
+                                                     block_table, table_stride, row_seq, positions, lambda, normalize, eps, \
+                                                     factor, gate, gate_dtype, gate_row, gate_act, out, out_dtype, n_heads,  \
+                                                     n_kv_heads, dim, vdim, page_tokens, window, keep_first, scale)
+  if (cache_dtype == kF32) {
+    if (maps == 1) BC4G_MAPS(float, 1); else BC4G_MAPS(float, 2);
+  } else if (cache_dtype == kBF16) {
+    if (maps == 1) BC4G_MAPS(bf16_t, 1); else BC4G_MAPS(bf16_t, 2);
+  } else {
+    return fail("attention_maps: unknown dtype %d", cache_dtype);
+  }
+#undef BC4G_MAPS
+  return check_launch("attention_maps");
+}

@@ -1,5 +1,5 @@
 // A norm that is added to the residual stream (the second norm of a layer whose sublayers are normed on both
-// sides), and the xIELU activation.  One instantiation per storage type; all arithmetic in float.
+// sides), the xIELU activation, and a gated unit with clamped branches.  One instantiation per storage type; all arithmetic in float.
 #include <math.h>
 
 #include "api.h"
@@ -58,6 +58,20 @@ __global__ void xielu_pieces_kernel(const uint4* __restrict__ in, uint4* __restr
   }
 }
 
+// out[t, i] = g sigmoid(slope g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit); gu [T, 2 I]: a row's
+// gates, then its ups.
+template <typename T>
+__global__ void clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ out, float limit, float slope, long total, int inter) {
+  const long stride = static_cast<long>(blockDim.x) * gridDim.x;
+  for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < total; i += stride) {
+    const long r = i / inter;
+    const int c = static_cast<int>(i - r * inter);
+    const float g = fminf(to_float(gu[r * 2 * inter + c]), limit);
+    const float u = fminf(fmaxf(to_float(gu[r * 2 * inter + inter + c]), -limit), limit);
+    out[i] = from_float<T>(g / (1.0f + expf(-slope * g)) * (u + 1.0f));
+  }
+}
+
 int grid_for(long total) {
   const long g = (total + kBlock - 1) / kBlock;
   return static_cast<int>(g < 1 ? 1 : (g > 65535 ? 65535 : g));
@@ -89,4 +103,15 @@ extern "C" int bc4g_xielu(const void* in, void* out, int dtype, const float* pq,
   else if (dtype == kBF16) xielu_kernel<bf16_t><<<grid_for(total), kBlock, 0, s>>>(static_cast<const bf16_t*>(in), static_cast<bf16_t*>(out), pq, total);
   else return fail("xielu: unknown dtype %d", dtype);
   return check_launch("xielu");
+}
+
+extern "C" int bc4g_clamped_glu(const void* gu, void* out, int dtype, float limit, float slope, int n_rows, int inter, void* stream) {
+  BC4G_REQUIRE(n_rows >= 0 && inter > 0 && gu && out && gu != out, "clamped_glu: bad arguments rows=%d I=%d", n_rows, inter);
+  if (n_rows == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const long total = static_cast<long>(n_rows) * inter;
+  if (dtype == kF32) clamped_glu_kernel<float><<<grid_for(total), kBlock, 0, s>>>(static_cast<const float*>(gu), static_cast<float*>(out), limit, slope, total, inter);
+  else if (dtype == kBF16) clamped_glu_kernel<bf16_t><<<grid_for(total), kBlock, 0, s>>>(static_cast<const bf16_t*>(gu), static_cast<bf16_t*>(out), limit, slope, total, inter);
+  else return fail("clamped_glu: unknown dtype %d", dtype);
+  return check_launch("clamped_glu");
 }

@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import ctypes
 import sys
-from ctypes import c_char_p, c_float, c_int, c_long, c_void_p
+from ctypes import c_char_p, c_double, c_float, c_int, c_long, c_void_p
 from typing import Optional
 
 from ..errors import KernelError
@@ -50,6 +50,17 @@ _SIGNATURES = {
     "bc4g_latent_prepare": [_P, _P, _I, _P, _F, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, c_long, c_long, _P],
     "bc4g_heads_gemm": [_P, _I, c_long, c_long, _P, _I, _P, _I, c_long, c_long, _I, _I, _I, _I, _P],
     "bc4g_attention_latent": [_P, _P, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
+    "bc4g_clamped_glu": [_P, _P, _I, _F, _F, _I, _I, _P],
+    "bc4g_streams_read": [_P, _P, _P, _P, _P, _P, _F, _P, _I, _I, _I, _I, _P],
+    "bc4g_streams_write": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "bc4g_streams_fill": [_P, _P, _I, _I, _I, _P],
+    "bc4g_rotary_table": [_P, _P, c_double, _P, _I, _I, _P],
+    "bc4g_heads_prepare": [_P, _I, c_long, _P, _P, _F, _P, _I, _F, _P, _I, c_long, _P, _I, c_long, c_long, c_long, _I, _I, _I, _P],
+    "bc4g_heads_finish": [_P, _P, _F, _F, _P, _I, c_long, _I, _P, _I, _I, _I, _I, _P],
+    "bc4g_decay_scan": [_P, _I, c_long, _F, _P, _I, c_long, _P, _I, c_long, _P, _P, _I, c_long, _P, _F, _P, _P, _P, _P, _P, _P, _P,
+                        _I, _I, _I, _I, _I, _I, _P],
+    "bc4g_attention_maps": [_P, c_long, _P, _P, _I, _P, _I, _P, _P, _F, _I, _F, _F, _P, _I, c_long, _I, _P, _I,
+                            _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _P],
     "bc4g_attention_latent_mfma": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
 }
 

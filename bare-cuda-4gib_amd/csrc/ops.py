@@ -1397,3 +1397,271 @@ def attention_latent_work(ctx, heads: int, rank: int, rot: int, window: int, ele
             pairs += new * cached + new * (new + 1) // 2
             keys += cached + new
     return 2.0 * pairs * heads * (2 * rank + rot), float(keys * (rank + rot) * elem)
+
+
+# ---- a residual stream in several copies, a pointwise norm, clamped gated units -----------------------------------------
+
+MAX_STREAMS = 8             # copies of the residual stream the kernels take
+
+
+def _streams(what: str, x: torch.Tensor):
+    if x.dtype != torch.float32 or x.dim() != 3 or not (1 <= x.shape[1] <= MAX_STREAMS):
+        raise KernelError(f"{what}: the stream must be float32 [T, copies (at most {MAX_STREAMS}), H], got {x.dtype} {tuple(x.shape)}")
+    return x.shape
+
+
+def streams_fill(x: torch.Tensor, copies: int) -> torch.Tensor:
+    """[T, H] float32 -> [T, copies, H], every copy equal to x."""
+    _dev("streams_fill", x)
+    if x.dtype != torch.float32 or x.dim() != 2 or copies < 1:
+        raise KernelError(f"streams_fill: x must be float32 [T, H], got {x.dtype} {tuple(x.shape)}")
+    t, hidden = x.shape
+    out = torch.empty((t, copies, hidden), dtype=torch.float32, device=x.device)
+    library.call("bc4g_streams_fill", _ptr(x), _ptr(out), t, copies, hidden, _stream(),
+                 cost=lambda: (0.0, 4.0 * t * hidden * (1 + copies)))
+    return out
+
+
+def streams_read(x: torch.Tensor, read: Optional[torch.Tensor], pointwise, out_dtype: torch.dtype,
+                 rows: Optional[torch.Tensor] = None, n_rows: Optional[int] = None) -> torch.Tensor:
+    """sum_s read[s] x[:, s] of the copies x [T, n, H] (``read`` None: every copy counts once), at ``rows`` only if
+    given; with ``pointwise`` = (alpha [1], g [H], b [H], out_scale) the norm (tanh(alpha u) g + b) out_scale of it."""
+    t, n, hidden = _streams("streams_read", x)
+    alpha, g, b, out_scale = pointwise if pointwise is not None else (None, None, None, 1.0)
+    _dev("streams_read", x, read, alpha, g, b, rows)
+    _f32("streams_read", "read", read, (n,))
+    _f32("streams_read", "alpha", alpha, (1,))
+    _f32("streams_read", "g", g, (hidden,))
+    _f32("streams_read", "b", b, (hidden,))
+    if rows is not None:
+        t = rows.numel() if n_rows is None else n_rows
+        _i32("streams_read", "rows", rows, t)
+    out = torch.empty((t, hidden), dtype=out_dtype, device=x.device)
+    library.call("bc4g_streams_read", _ptr(x), _ptr(rows), _ptr(read), _ptr(alpha), _ptr(g), _ptr(b), float(out_scale), _ptr(out),
+                 _code(out, "streams_read"), t, n, hidden, _stream(),
+                 cost=lambda: (2.0 * t * hidden * (n + 2), t * hidden * (4 * n + out.element_size())))
+    return out
+
+
+def streams_write(x: torch.Tensor, y: torch.Tensor, mix: torch.Tensor, write: torch.Tensor,
+                  next_read: Optional[torch.Tensor] = None, pointwise=None, out_dtype: Optional[torch.dtype] = None):
+    """x'[:, t] = sum_s mix[s, t] x[:, s] + write[t] y in place on the copies x [T, n, H] (y float32 [T, H]); with
+    ``next_read`` also returns the next reader's input from the new copies (see streams_read; the norm's out_scale is 1)."""
+    t, n, hidden = _streams("streams_write", x)
+    alpha, g, b, _ = pointwise if pointwise is not None else (None, None, None, 1.0)
+    _dev("streams_write", x, y, mix, write, next_read, alpha, g, b)
+    _f32("streams_write", "y", y, (t, hidden))
+    _f32("streams_write", "mix", mix, (n, n))
+    _f32("streams_write", "write", write, (n,))
+    _f32("streams_write", "next_read", next_read, (n,))
+    _f32("streams_write", "alpha", alpha, (1,))
+    _f32("streams_write", "g", g, (hidden,))
+    _f32("streams_write", "b", b, (hidden,))
+    out = None
+    if next_read is not None:
+        out = torch.empty((t, hidden), dtype=out_dtype or torch.float32, device=x.device)
+    library.call("bc4g_streams_write", _ptr(x), _ptr(y), _ptr(mix), _ptr(write), _ptr(next_read), _ptr(alpha), _ptr(g), _ptr(b),
+                 _ptr(out), _code(out, "streams_write") if out is not None else F32, t, n, hidden, _stream(),
+                 cost=lambda: (2.0 * t * hidden * n * (n + 2), t * hidden * (8 * n + 4 + (out.element_size() if out is not None else 0))))
+    return out
+
+
+def clamped_glu(gu: torch.Tensor, limit: float, slope: float) -> torch.Tensor:
+    """gu [T, 2I] (a row's gates, then its ups) -> g sigmoid(slope g) (u + 1) with g = min(gate, limit),
+    u = clamp(up, -limit, limit), [T, I]."""
+    _dev("clamped_glu", gu)
+    if gu.dim() != 2 or gu.shape[1] % 2:
+        raise KernelError(f"clamped_glu: input must be [T, 2I], got {tuple(gu.shape)}")
+    t, inter = gu.shape[0], gu.shape[1] // 2
+    out = torch.empty((t, inter), dtype=gu.dtype, device=gu.device)
+    library.call("bc4g_clamped_glu", _ptr(gu), _ptr(out), _code(gu, "clamped_glu"), float(limit), float(slope), t, inter, _stream(),
+                 cost=lambda: (8.0 * t * inter, 3 * t * inter * gu.element_size()))
+    return out
+
+
+# ---- heads: rotation tables, preparation, finishing; linear attention with a decayed state; attention with two maps -----
+
+HEADS_MAX_DIM = 256         # elements of a head that heads_prepare, heads_finish, decay_scan and attention_maps take
+DECAY_SCAN_CHUNK = 64       # rows of a request that one workgroup of the scan walks
+
+ACT_NONE, ACT_SILU, ACT_SIGMOID = 0, 1, 2
+
+
+def _part_of_rows(what: str, name: str, t: torch.Tensor, width: int) -> int:
+    """The row stride of a [T, >= width] tensor on the GPU that may be a part of one product's wider rows."""
+    if not t.is_cuda or t.dim() != 2 or t.shape[1] < width or (t.shape[1] > 1 and t.stride(1) != 1) or t.stride(0) < t.shape[1]:
+        raise KernelError(f"{what}: {name} must be [T, {width}] on the GPU with a row's elements side by side, got shape "
+                          f"{tuple(t.shape)} with strides {t.stride()} on {t.device}")
+    return t.stride(0)
+
+
+def rotary_table(positions: torch.Tensor, freqs: torch.Tensor, amplitude: float = 1.0) -> torch.Tensor:
+    """[T, half, 2] float32: cos and sin of positions[t] * freqs[i] (freqs float64 [half] on the device), times
+    ``amplitude``; the angles are worked out in double."""
+    _dev("rotary_table", positions, freqs)
+    n, half = positions.numel(), freqs.numel()
+    _i32("rotary_table", "positions", positions, n)
+    if freqs.dtype != torch.float64 or freqs.dim() != 1 or half < 1:
+        raise KernelError(f"rotary_table: freqs must be float64 [half], got {freqs.dtype} {tuple(freqs.shape)}")
+    table = torch.empty((n, half, 2), dtype=torch.float32, device=positions.device)
+    library.call("bc4g_rotary_table", _ptr(positions), _ptr(freqs), float(amplitude), _ptr(table), n, half, _stream(),
+                 cost=lambda: (40.0 * n * half, 8.0 * n * half))
+    return table
+
+
+def heads_prepare(x: torch.Tensor, heads: int, dim: int, out: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
+                  norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0, table: Optional[torch.Tensor] = None,
+                  factor: float = 1.0, slot_map: Optional[torch.Tensor] = None, page_tokens: int = 0) -> torch.Tensor:
+    """Every head of x [T, heads * dim] (may be a part of wider rows): + bias, RMS norm over the head with
+    ``norm_weight`` [dim], rotation by ``table`` [T, half, 2] (element i with element i + half), times ``factor``.
+    ``out``: [T, heads, dim] (float32 or bfloat16), or with ``slot_map`` a cache [pages, heads, page_tokens, dim] whose
+    slot page * page_tokens + offset receives the row."""
+    _dev("heads_prepare", bias, norm_weight, table, out, slot_map)
+    in_row = _part_of_rows("heads_prepare", "x", x, heads * dim)
+    t = x.shape[0]
+    _f32("heads_prepare", "bias", bias, (heads * dim,))
+    _f32("heads_prepare", "norm_weight", norm_weight, (dim,))
+    half = 0
+    if table is not None:
+        half = table.shape[1]
+        _f32("heads_prepare", "table", table, (t, half, 2))
+    if dim > HEADS_MAX_DIM or 2 * half > dim:
+        raise KernelError(f"heads_prepare: heads of {dim} elements (at most {HEADS_MAX_DIM}) with {half} rotated pairs")
+    if slot_map is not None:
+        _i32("heads_prepare", "slot_map", slot_map, t)
+        if out.dim() != 4 or tuple(out.shape[1:]) != (heads, page_tokens, dim):
+            raise KernelError(f"heads_prepare: the cache must be [pages, {heads}, {page_tokens}, {dim}], got {tuple(out.shape)}")
+        page_stride, head_stride, token_stride, out_row = heads * page_tokens * dim, page_tokens * dim, dim, 0
+    else:
+        if tuple(out.shape) != (t, heads, dim):
+            raise KernelError(f"heads_prepare: out must be [{t}, {heads}, {dim}], got {tuple(out.shape)}")
+        page_stride = head_stride = token_stride = 0
+        out_row = heads * dim
+    library.call("bc4g_heads_prepare", _ptr(x), _code(x, "heads_prepare"), in_row, _ptr(bias), _ptr(norm_weight), float(eps),
+                 _ptr(table), half, float(factor), _ptr(out), _code(out, "heads_prepare"), out_row, _ptr(slot_map), page_tokens,
+                 page_stride, head_stride, token_stride, t, heads, dim, _stream(),
+                 cost=lambda: (8.0 * t * heads * dim, t * heads * dim * (x.element_size() + out.element_size())))
+    return out
+
+
+def heads_finish(o: torch.Tensor, out_dtype: torch.dtype, *, weight: Optional[torch.Tensor] = None, eps: float = 0.0,
+                 factor: float = 1.0, gate: Optional[torch.Tensor] = None, act: int = ACT_NONE) -> torch.Tensor:
+    """o float32 [T, heads, vdim] -> o / sqrt(mean(o^2) + eps) (* weight [vdim]) * factor * act(gate) per head, as
+    [T, heads * vdim] in ``out_dtype``; gate [T, heads * vdim] may be a part of wider rows."""
+    _dev("heads_finish", o, weight)
+    if o.dtype != torch.float32 or o.dim() != 3 or o.shape[2] > HEADS_MAX_DIM:
+        raise KernelError(f"heads_finish: o must be float32 [T, heads, vdim <= {HEADS_MAX_DIM}], got {o.dtype} {tuple(o.shape)}")
+    t, heads, vdim = o.shape
+    _f32("heads_finish", "weight", weight, (vdim,))
+    gate_row = _part_of_rows("heads_finish", "gate", gate, heads * vdim) if gate is not None else 0
+    if gate is not None and gate.shape[0] != t:
+        raise KernelError(f"heads_finish: gate has {gate.shape[0]} rows, o {t}")
+    out = torch.empty((t, heads * vdim), dtype=out_dtype, device=o.device)
+    library.call("bc4g_heads_finish", _ptr(o), _ptr(weight), float(eps), float(factor), _ptr(gate),
+                 _code(gate, "heads_finish") if gate is not None else F32, gate_row, int(act), _ptr(out), _code(out, "heads_finish"),
+                 t, heads, vdim, _stream(),
+                 cost=lambda: (10.0 * t * heads * vdim, t * heads * vdim * (4 + 2 * out.element_size())))
+    return out
+
+
+def decay_scan_chunks(batch) -> Tuple[list, int]:
+    """(first chunk of every request among all chunks of the requests that bring two chunks or more, how many such
+    chunks there are) for a step's HostBatch."""
+    base, total = [], 0
+    for s in range(batch.n_seqs):
+        n = -(-int(batch.seq_start[s + 1] - batch.seq_start[s]) // DECAY_SCAN_CHUNK)
+        base.append(total)
+        if n >= 2:
+            total += n
+    return base, total
+
+
+def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.Tensor, ctx, heads: int, dim: int, vdim: int, *,
+               head_decay: Optional[torch.Tensor] = None, z: Optional[torch.Tensor] = None, z_bias: Optional[torch.Tensor] = None,
+               inv_tau: float = 1.0, q_scale: float = 1.0, chunk_base: Optional[torch.Tensor] = None, n_chunks: int = 0) -> torch.Tensor:
+    """S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T (q_t q_scale) per request and head over a step's rows; q, k
+    [T, heads * dim], v [T, heads * vdim] (float32 or bfloat16, each may be a part of wider rows); state float32
+    [slots, heads, dim, vdim] is read and left.  a_t = head_decay[head] (float32 [heads]) or, with gate logits z
+    [T, heads * dim], sigmoid(z + z_bias)^inv_tau.  ``chunk_base`` (int32 [S] on the device) and ``n_chunks``:
+    see decay_scan_chunks -- needed when a request brings more than DECAY_SCAN_CHUNK rows.  Returns float32 [T, heads, vdim]."""
+    _dev("decay_scan", head_decay, z_bias, state, chunk_base)
+    t = q.shape[0]
+    q_row = _part_of_rows("decay_scan", "q", q, heads * dim)
+    k_row = _part_of_rows("decay_scan", "k", k, heads * dim)
+    v_row = _part_of_rows("decay_scan", "v", v, heads * vdim)
+    z_row = _part_of_rows("decay_scan", "z", z, heads * dim) if z is not None else 0
+    if k.shape[0] != t or v.shape[0] != t or (z is not None and z.shape[0] != t):
+        raise KernelError("decay_scan: q, k, v and z must have the same number of rows")
+    if (head_decay is None) == (z is None):
+        raise KernelError("decay_scan: either a decay per head or gate logits per token")
+    _f32("decay_scan", "head_decay", head_decay, (heads,))
+    _f32("decay_scan", "z_bias", z_bias, (heads * dim,))
+    if (state.dtype != torch.float32 or state.dim() != 4 or tuple(state.shape[1:]) != (heads, dim, vdim)
+            or max(ctx.seq_slots, default=0) >= state.shape[0]):
+        raise KernelError(f"decay_scan: state must be float32 [slots, {heads}, {dim}, {vdim}] with a row for every slot of the step")
+    if dim > HEADS_MAX_DIM:
+        raise KernelError(f"decay_scan: {dim} key channels a head are beyond the kernel's {HEADS_MAX_DIM}")
+    _check_grouping("decay_scan", ctx, t)
+    most = max(int(ctx.seq_start[s + 1] - ctx.seq_start[s]) for s in range(ctx.n_seqs))
+    chunk_state = chunk_decay = None
+    if most > DECAY_SCAN_CHUNK:
+        if chunk_base is None or n_chunks < 2:
+            raise KernelError("decay_scan: a request brings several chunks of rows and the chunks' places are not given")
+        _i32("decay_scan", "chunk_base", chunk_base, ctx.n_seqs)
+        chunk_state = torch.empty((n_chunks, heads, dim, vdim), dtype=torch.float32, device=state.device)
+        chunk_decay = torch.empty((n_chunks, heads, dim), dtype=torch.float32, device=state.device)
+    out = torch.empty((t, heads, vdim), dtype=torch.float32, device=state.device)
+    passes = 2 if most > DECAY_SCAN_CHUNK else 1
+    library.call("bc4g_decay_scan", _ptr(q), _code(q, "decay_scan"), q_row, float(q_scale), _ptr(k), _code(k, "decay_scan"), k_row,
+                 _ptr(v), _code(v, "decay_scan"), v_row, _ptr(head_decay), _ptr(z), _code(z, "decay_scan") if z is not None else F32,
+                 z_row, _ptr(z_bias), float(inv_tau), _ptr(out), _ptr(state), _ptr(chunk_state), _ptr(chunk_decay),
+                 _ptr(ctx.seq_start_dev), _ptr(ctx.seq_slots_dev), _ptr(chunk_base), t, ctx.n_seqs, most, heads, dim, vdim, _stream(),
+                 cost=lambda: (passes * 4.0 * t * heads * dim * vdim,
+                               t * heads * (2 * dim * q.element_size() + vdim * (v.element_size() + 4))
+                               + 8.0 * ctx.n_seqs * heads * dim * vdim))
+    return out
+
+
+def attention_maps(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor, ctx, out_dtype: torch.dtype,
+                   n_heads: int, n_kv_heads: int, maps: int, dim: int, vdim: int, window: int, keep_first: int, scale: float, *,
+                   lam: float = 0.0, normalize: bool = False, eps: float = 0.0, factor: float = 1.0,
+                   gate: Optional[torch.Tensor] = None, act: int = ACT_SIGMOID) -> torch.Tensor:
+    """Softmax attention with ``maps`` (1 or 2) score maps per query head over the same values: q float32
+    [T, n_heads, maps, dim]; keys [pages, n_kv_heads * maps, page_tokens, dim], values [pages, n_kv_heads, page_tokens, vdim].
+    A row at position p sees key j <= p if p - j < window or j < keep_first (window 0: every key).  o = a1 - lam a2,
+    with ``normalize`` divided by sqrt(mean(o^2) + eps) over the head, times ``factor`` and act(gate); [T, n_heads * vdim]."""
+    _dev("attention_maps", q, k_cache, v_cache, block_table)
+    t = q.shape[0]
+    if q.dtype != torch.float32 or tuple(q.shape) != (t, n_heads, maps, dim):
+        raise KernelError(f"attention_maps: q must be float32 [T, {n_heads}, {maps}, {dim}], got {q.dtype} {tuple(q.shape)}")
+    if k_cache.dim() != 4 or v_cache.dim() != 4 or k_cache.dtype != v_cache.dtype:
+        raise KernelError("attention_maps: caches must be [pages, heads, page_tokens, size] of one dtype")
+    pages, _, page_tokens, _ = k_cache.shape
+    if tuple(k_cache.shape[1:]) != (n_kv_heads * maps, page_tokens, dim) or tuple(v_cache.shape) != (pages, n_kv_heads, page_tokens, vdim):
+        raise KernelError(f"attention_maps: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} do not fit {n_kv_heads} key/value heads, "
+                          f"{maps} maps of {dim}, values of {vdim}")
+    if ctx.n_tokens != t or block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.shape[0] < ctx.n_seqs:
+        raise KernelError("attention_maps: the block table does not fit the step")
+    _i32("attention_maps", "row_seq", ctx.row_seq, t)
+    _i32("attention_maps", "positions", ctx.positions, t)
+    gate_row = _part_of_rows("attention_maps", "gate", gate, n_heads * vdim) if gate is not None else 0
+    out = torch.empty((t, n_heads * vdim), dtype=out_dtype, device=q.device)
+
+    def cost():
+        keys = pairs = 0
+        for s in range(ctx.n_seqs):
+            cached, new = int(ctx.seq_ctx[s]), int(ctx.seq_start[s + 1] - ctx.seq_start[s])
+            if window > 0:
+                pairs += sum(min(window + keep_first, cached + i + 1) for i in range(new))
+                keys += min(cached + new, window + keep_first + new - 1)
+            else:
+                pairs += new * cached + new * (new + 1) // 2
+                keys += cached + new
+        return (2.0 * pairs * n_heads * maps * (dim + vdim),
+                keys * n_kv_heads * (maps * dim + vdim) * k_cache.element_size() + t * n_heads * (4 * maps * dim + vdim * out.element_size()))
+    library.call("bc4g_attention_maps", _ptr(q), n_heads * maps * dim, _ptr(k_cache), _ptr(v_cache), _code(k_cache, "attention_maps"),
+                 _ptr(block_table), block_table.stride(0), _ptr(ctx.row_seq), _ptr(ctx.positions), float(lam), 1 if normalize else 0,
+                 float(eps), float(factor), _ptr(gate), _code(gate, "attention_maps") if gate is not None else F32, gate_row, int(act),
+                 _ptr(out), _code(out, "attention_maps"), t, n_heads, n_kv_heads, maps, dim, vdim, page_tokens, int(window),
+                 int(keep_first), float(scale), _stream(), cost=cost)
+    return out

@@ -58,6 +58,7 @@ class Model:
         self.vocab_size = spec.vocab_size
         self.hidden_size = spec.hidden_size
         self.max_seq_len = spec.max_seq_len
+        self.streams = int(getattr(spec, "streams", 1))
         self.rt: Optional[Runtime] = None
 
     def all_parts(self) -> List[Part]:
@@ -169,7 +170,7 @@ class Model:
         layer's activations are given back before the next runs), and the float logits."""
         layer = max((part.working_bytes_per_row(elem) for part in self.layers), default=0.0)
         head = self.final_norm.part.working_bytes_per_row(elem) + self.hidden_size * elem
-        per_row = self.hidden_size * (4 + 4 + elem) + self.embedding.part.working_bytes_per_row(elem) + layer
+        per_row = self.hidden_size * (4 * self.streams + 4 + elem) + self.embedding.part.working_bytes_per_row(elem) + layer
         return int(rows * per_row + n_logits * (head + 4 * self.vocab_size))
 
     # ---- forward ------------------------------------------------------------
@@ -177,6 +178,9 @@ class Model:
         """Run the batch through every schedule entry; float32 logits at the
         wanted rows ([n_logits, vocab]), or None if none are wanted."""
         x = self.embedding.part.forward(ctx)
+        if self.streams > 1:            # the stream in copies, [T, streams, H]: every copy starts as the embedding
+            from ..csrc import ops
+            x = ops.streams_fill(x, self.streams)
         ctx.handoff.end_step()
         for i, e in enumerate(self.schedule):
             layer = self.layers[e.layer]
@@ -187,6 +191,12 @@ class Model:
         if ctx.n_logits == 0:
             return None
         norm, head = self.final_norm.part, self.head.part
+        if x.dim() == 3 and not hasattr(norm, "pointwise"):
+            # a norm that reads whole rows gets the sum of the copies at the wanted rows (one that works element by
+            # element sums them itself)
+            from ..csrc import ops
+            x = ops.streams_read(x, None, None, torch.float32, rows=ctx.logit_rows, n_rows=ctx.n_logits)
+            return head.forward(norm.forward(x, ctx))
         if getattr(head, "accepts_lazy_norm", False):
             return head.forward(Normed(x, norm, ctx, rows=ctx.logit_rows, n_rows=ctx.n_logits))
         return head.forward(norm.forward(x, ctx, rows=ctx.logit_rows, n_rows=ctx.n_logits))

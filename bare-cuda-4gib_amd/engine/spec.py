@@ -56,3 +56,6 @@ class ModelSpec:
     schedule: List[ScheduleEntry]
     final_norm: PartSpec
     head: PartSpec
+    # copies of the residual stream that the layers keep side by side, [T, streams, H] (1: the plain stream [T, H]); all
+    # start as the embedding's output, and the model's last norm reads their sum
+    streams: int = 1

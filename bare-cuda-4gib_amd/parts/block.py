@@ -7,6 +7,7 @@ from ..cache.specs import Bundle
 from ..csrc import ops
 from .base import Part, register_part
 from .lazy import Normed
+from .streams import StreamReader
 
 
 class PreNormBlock(Part):
@@ -104,5 +105,57 @@ class SandwichBlock(Part):
         return y.tensor if isinstance(y, ops.Fresh) else y
 
 
+class HyperBlock(Part):
+    """Pre-norm sublayers on a residual stream kept in several copies x [T, n, H]: each sublayer reads one weighted sum
+    of the copies through its norm and writes all copies at once (parts.streams.HyperConnection):
+    y = mixer(norm1(read1(x))); x = write1(x, y); then the same with the feed-forward, if the layer has one.  The read
+    of whoever comes next -- this layer's feed-forward, the next layer's mixer -- is made by the write before it."""
+    category = "block"
+    graph_safe = True     # launches kernels only: may run inside a captured graph
+
+    def __init__(self, mixer, mixer_norm, mixer_conn, ffn=None, ffn_norm=None, ffn_conn=None):
+        self.mixer, self.mixer_norm, self.mixer_conn = mixer, mixer_norm, mixer_conn
+        self.ffn, self.ffn_norm, self.ffn_conn = ffn, ffn_norm, ffn_conn
+        self.mixer_reader = StreamReader(mixer_conn, mixer_norm)
+        self.ffn_reader = StreamReader(ffn_conn, ffn_norm) if ffn is not None else None
+
+    def children(self):
+        parts = [self.mixer_conn, self.mixer_norm, self.mixer, self.ffn_conn, self.ffn_norm, self.ffn]
+        return [p for p in parts if p is not None]
+
+    @staticmethod
+    def _sum_for(part, x):
+        """What the part adds its output [T, H] to: nothing yet for a part whose output is one last product, else a cleared buffer."""
+        if getattr(part, "adds_one_product", False):
+            return ops.Fresh()
+        return torch.zeros((x.shape[0], x.shape[2]), dtype=torch.float32, device=x.device)
+
+    def first_reader(self, n_rows: int):
+        """What the entry before may prepare: this block's first input (a reader that takes no parts of an RMSNorm)."""
+        return self.mixer_reader, False
+
+    def forward(self, x, ctx, cache, writes: bool = True) -> None:
+        handoff = ctx.handoff
+        h = handoff.take(self.mixer_reader)
+        if h is None:
+            h = self.mixer_conn.read(x, self.mixer_norm, ctx)
+        following = handoff.next_entry[0] if handoff.next_entry is not None else None
+        if not isinstance(following, StreamReader) or following.connection.streams != self.mixer_conn.streams:
+            following = None
+        y = self._sum_for(self.mixer, x)
+        self.mixer.forward(h, ctx, cache, y, writes)
+        if self.ffn is None:
+            last_conn = self.mixer_conn
+        else:
+            h = self.mixer_conn.write(x, SandwichBlock._sum_of(y), self.ffn_reader, ctx)
+            y = self._sum_for(self.ffn, x)
+            self.ffn.forward(h, ctx, y)
+            last_conn = self.ffn_conn
+        made = last_conn.write(x, SandwichBlock._sum_of(y), following, ctx)
+        if following is not None:
+            handoff.leave(following, made)
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "hyper", HyperBlock)
 register_part("block", "sandwich", SandwichBlock)

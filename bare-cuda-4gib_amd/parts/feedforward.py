@@ -81,5 +81,36 @@ class DenseXIELU(Part):
         linear(ops.xielu(z, self.pq, out=z), self.w_down, accumulate_into=residual, ctx=ctx)
 
 
+class ClampedGLU(Part):
+    """x += Wd (g sigmoid(slope g) (u + 1)) with g = min(Wg h, limit) and u = clamp(Wu h, -limit, limit), no biases."""
+    category = "feedforward"
+    graph_safe = True     # launches kernels only: may run inside a captured graph
+    adds_one_product = True   # the output is one last product through linear(): a block may hand it ops.Fresh
+
+    def __init__(self, hidden_size: int, intermediate_size: int, limit: float, slope: float = 1.702):
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.limit, self.slope = float(limit), float(slope)
+        self.w_gu = self.w_down = None
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        h, i = self.hidden_size, self.intermediate_size
+        return {"gate": WeightSpec((i, h)), "up": WeightSpec((i, h)), "down": WeightSpec((h, i))}
+
+    def bind(self, tensors, rt) -> None:
+        # one product for gate and up: the gates' rows, then the ups'
+        self.w_gu = ops.StreamedWeight(torch.cat([tensors["gate"], tensors["up"]], dim=0).contiguous())
+        self.w_down = ops.StreamedWeight(tensors["down"])
+        self.act_dtype = rt.act_dtype
+
+    def step_work(self, batch, rows: int, elem: int):
+        flops, nbytes = super().step_work(batch, rows, elem)
+        return flops + 8.0 * rows * self.intermediate_size, nbytes
+
+    def forward(self, h, ctx, residual) -> None:
+        gu = linear(h, self.w_gu, out_dtype=self.act_dtype)
+        linear(ops.clamped_glu(gu, self.limit, self.slope), self.w_down, accumulate_into=residual, ctx=ctx)
+
+
 register_part("feedforward", "swiglu", SwiGLU)
+register_part("feedforward", "clamped_glu", ClampedGLU)
 register_part("feedforward", "dense_xielu", DenseXIELU)

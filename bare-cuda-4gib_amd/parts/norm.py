@@ -44,4 +44,33 @@ class RMSNorm(Part):
         return ops.rmsnorm(x, self.weight, self.eps, self.out_dtype, rows=rows, n_rows=n_rows)
 
 
+class DynamicTanh(Part):
+    """y = (tanh(alpha x) * w + b) * out_scale, element by element: a norm that computes no mean and no variance.
+    ``alpha`` is one number stored beside the weight.  Arithmetic is float32.  The input may be the residual stream
+    in several copies, [T, n, H]: the norm is then taken of their sum."""
+    category = "norm"
+    graph_safe = True
+
+    def __init__(self, size: int, out_scale: float = 1.0):
+        self.size, self.out_scale = int(size), float(out_scale)
+        self.weight = self.bias = self.alpha = None
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        return {"weight": WeightSpec((self.size,), kind="vector", init="ones"), "b": WeightSpec((self.size,), kind="vector"),
+                "alpha": WeightSpec((), kind="vector", init="ones")}
+
+    def bind(self, tensors, rt) -> None:
+        f32 = lambda name: tensors[name].to(torch.float32).reshape(-1).contiguous()      # noqa: E731
+        self.weight, self.bias, self.alpha = f32("weight"), f32("b"), f32("alpha")
+        self.out_dtype = rt.act_dtype
+
+    def pointwise(self):
+        """What a kernel that has the norm's input in registers needs to apply it: (alpha [1], w, b, out_scale)."""
+        return self.alpha, self.weight, self.bias, self.out_scale
+
+    def forward(self, x: torch.Tensor, ctx=None, rows=None, n_rows=None) -> torch.Tensor:
+        return ops.streams_read(x if x.dim() == 3 else x.unsqueeze(1), None, self.pointwise(), self.out_dtype, rows=rows, n_rows=n_rows)
+
+
 register_part("norm", "rmsnorm", RMSNorm)
+register_part("norm", "dynamic_tanh", DynamicTanh)

@@ -1,6 +1,8 @@
 """Position encodings applied to queries and keys before keys are cached."""
 from __future__ import annotations
 
+import math
+
 from ..errors import ConfigError
 from .base import Part, register_part
 
@@ -10,19 +12,59 @@ class Rotary(Part):
     i + dim/2): inv_freq_i = theta^(-2i/dim), angle = position * inv_freq_i,
     (lo, hi) -> (lo cos - hi sin, hi cos + lo sin), angles in float
     (reference: engine/kernels/rope.cu:44-53).  ``dim`` may be smaller than the
-    head size; the remaining elements pass through."""
+    head size; the remaining elements pass through.
+
+    ``scaling`` (factor F, original L, fast, slow) stretches the slow pairs for contexts beyond L: with
+    e(t) = dim ln(L / (2 pi t)) / (2 ln theta), lo = max(floor(e(fast)), 0), hi = min(ceil(e(slow)), dim - 1) and
+    r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i turns with inv_freq_i / F * r_i + inv_freq_i (1 - r_i), and
+    cosines and sines are multiplied by 0.1 ln F + 1.  The kernels that rotate inside a product take no scaling
+    (``fused()`` is None then); ``table(ctx)`` gives every row's cosines and sines to whoever rotates by a table."""
     category = "position"
     graph_safe = True     # launches kernels only: may run inside a captured graph
 
-    def __init__(self, theta: float, dim: int):
+    def __init__(self, theta: float, dim: int, scaling=None):
         if dim <= 0 or dim % 2:
             raise ConfigError(f"rotary: dim must be positive and even, got {dim}")
         if theta <= 0:
             raise ConfigError(f"rotary: theta must be positive, got {theta}")
         self.theta, self.dim = float(theta), int(dim)
+        self.scaling = None
+        if scaling is not None:
+            try:
+                self.scaling = tuple(float(scaling[k]) for k in ("factor", "original", "fast", "slow"))
+            except (KeyError, TypeError, ValueError):
+                raise ConfigError(f"rotary: scaling must give factor, original, fast and slow, got {scaling!r}") from None
+            if min(self.scaling) <= 0 or self.theta == 1.0:
+                raise ConfigError(f"rotary: scaling {scaling!r} with theta {theta}: every number must be positive, theta not 1")
+        self._freqs = None
 
     def fused(self):
-        return self.dim, self.theta
+        return (self.dim, self.theta) if self.scaling is None else None
+
+    def apply(self, qkv, ctx, n_heads, n_kv_heads, head_dim):
+        raise ConfigError("rotary: scaled frequencies are applied by a table (table(ctx)); this mixer rotates inside its product")
+
+    def frequencies(self):
+        """(what pair i turns by per position, for i < dim / 2, as Python floats; the factor on cosines and sines)."""
+        half = self.dim // 2
+        freqs = [self.theta ** (-2.0 * i / self.dim) for i in range(half)]
+        if self.scaling is None:
+            return freqs, 1.0
+        factor, original, fast, slow = self.scaling
+        where = lambda t: self.dim * math.log(original / (2.0 * math.pi * t)) / (2.0 * math.log(self.theta))      # noqa: E731
+        lo, hi = max(math.floor(where(fast)), 0), min(math.ceil(where(slow)), self.dim - 1)
+        ramp = [min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0) for i in range(half)]
+        return [f / factor * r + f * (1.0 - r) for f, r in zip(freqs, ramp)], 0.1 * math.log(factor) + 1.0
+
+    def table(self, ctx):
+        """[T, dim / 2, 2] float32: every row's cosines and sines, made once a step for all layers that rotate alike."""
+        import torch
+        from ..csrc import ops
+        freqs, amplitude = self.frequencies()
+        if self._freqs is None or self._freqs.device != ctx.positions.device:
+            self._freqs = torch.tensor(freqs, dtype=torch.float64, device=ctx.positions.device)
+        return ctx.shared(("rotary_table", self.dim, self.theta, self.scaling),
+                          lambda: ops.rotary_table(ctx.positions, self._freqs, amplitude))
 
 
 class NoPosition(Part):

@@ -30,12 +30,18 @@ class WeightSpec:
     scale and the like), ``table`` (rows looked up by index) or ``int_table``
     (integer table, kept as int32).  ``init`` is what the random-weights mode
     writes: ``normal`` (N(0, std)) or ``ones``.  An ``optional`` tensor may be
-    absent (a tied output head).
+    absent (a tied output head).  A dimension of -1 in ``shape`` is a size that only the stored tensor gives.
     """
     shape: Tuple[int, ...]
     kind: str = "matrix"
     init: str = "normal"
     optional: bool = False
+
+
+def _shape_fits(found: Tuple[int, ...], wanted: Tuple[int, ...]) -> bool:
+    """Whether a stored shape is the expected one; a dimension expected as -1 is a size that the configuration does
+    not give and the part reads from the tensor when it is bound."""
+    return len(found) == len(wanted) and all(w == -1 or f == w for f, w in zip(found, wanted))
 
 
 def _kept_dtype_ok(spec: WeightSpec, t: torch.Tensor) -> bool:
@@ -65,7 +71,7 @@ def load_weights(model_dir: str, expected: Dict[str, WeightSpec],
                 missing.append(name)
             continue
         f, n = available[name]
-        if tuple(f.shape(n)) != tuple(spec.shape):
+        if not _shape_fits(tuple(f.shape(n)), tuple(spec.shape)):
             wrong.append(f"{name}: file has {list(f.shape(n))}, the configuration needs {list(spec.shape)}")
         elif spec.kind == "int_table" and not f.stored_dtype(n).startswith(("I", "U")):
             wrong.append(f"{name}: file has dtype {f.stored_dtype(n)}, an integer table is needed")
