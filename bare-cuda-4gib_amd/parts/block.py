@@ -136,6 +136,8 @@ class HyperBlock(Part):
 
     def forward(self, x, ctx, cache, writes: bool = True) -> None:
         handoff = ctx.handoff
+        if x.dim() == 2:              # a plain stream is one copy
+            x = x.unsqueeze(1)
         h = handoff.take(self.mixer_reader)
         if h is None:
             h = self.mixer_conn.read(x, self.mixer_norm, ctx)
