@@ -73,6 +73,30 @@ MAMENEX_SIZES = {
            dict(TINYLLAMA, tie_word_embeddings=True, max_position_embeddings=8192, hidden_size=4096, num_hidden_layers=6, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
                 intermediate_size=9600)),
 }
+
+
+def nagezen_shape(width, layers, heads, kv_heads, dim, vdim, ff, streams=4, window=1024, keep_first=4, vocab=32000):
+    """A Nagezen configuration of real layer sizes: every third layer differential attention (two maps of ``dim`` a head)
+    with a window, the others gated linear attention and retention in turn (states of dim x vdim a head), all with the
+    clamped gated feed-forward, the stream in ``streams`` copies."""
+    mlp = dict(kind="dense", ff=ff, limit=7.0)
+    att = dict(type="attention", mlp=mlp, mixer=dict(
+        heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, diff=0.5, scale=dim ** -0.5, mask=dict(size=window, keep_first=keep_first),
+        rot=dict(base=10000.0, dims=dim, scaling=dict(factor=4.0, original=2048, fast=32.0, slow=1.0))))
+    gla = dict(type="gla", mlp=mlp, mixer=dict(heads=heads, dim=dim, vdim=vdim, tau=16.0, rank=16))
+    ret = dict(type="retention", mlp=mlp, mixer=dict(heads=heads, dim=dim, vdim=vdim, rot=dict(base=10000.0, dims=dim),
+                                                     decay=[1.0 - 2.0 ** -(5 + 4 * a // heads) for a in range(heads)]))
+    order = [att if i % 3 == 0 else (gla if i % 3 == 1 else ret) for i in range(layers)]
+    return dict(architecture="Nagezen", vocab=vocab, width=width, streams=streams, logit_scale=1.0, norm=dict(eps=1e-6), layers=order)
+
+
+# --only nagezen: the design at a few sizes that resemble a real model's layers, each beside the Mamenex decoder (the
+# other design here whose layers keep a state per request beside pages per token) of the same width, depth and head count.
+NAGEZEN_SIZES = {
+    "1k": (nagezen_shape(1024, 6, 8, 2, 64, 128, 2752), MAMENEX_SIZES["1k"][0]),
+    "2k": (nagezen_shape(2048, 6, 16, 4, 64, 128, 5504), MAMENEX_SIZES["2k"][0]),
+    "4k": (nagezen_shape(4096, 6, 32, 8, 64, 128, 9600), MAMENEX_SIZES["4k"][0]),
+}
 BASELINE_DECODE_B1 = 77.3                   # the reference's only FP16 decode number (batch 1, RTX 3050)
 
 
@@ -240,14 +264,14 @@ def kernel_table(model, cfg, prefill_tokens, batch, context, dtype):
     return out
 
 
-def run_mamenex(size, args):
-    """Prefill and decode of the design at one size beside the Llama decoder of equal size; with --kernels the
-    per-kernel tables of both."""
+def run_mamenex(size, args, only="mamenex", names=("mamenex", "llama"), sizes=None):
+    """Prefill and decode of a design at one size beside another decoder of equal size (Mamenex beside Llama, Nagezen
+    beside Mamenex); with --kernels the per-kernel tables of both."""
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     elem = 2 if args.dtype == "bf16" else 4
-    line = {"only": "mamenex", "size": size, "dtype": args.dtype, "prefill_tokens": args.prefill_tokens, "batch": args.batch,
+    line = {"only": only, "size": size, "dtype": args.dtype, "prefill_tokens": args.prefill_tokens, "batch": args.batch,
             "prompt_len": args.prompt_len}
-    for name, shape in zip(("mamenex", "llama"), MAMENEX_SIZES[size]):
+    for name, shape in zip(names, (sizes or MAMENEX_SIZES)[size]):
         import torch
         model, cfg = build_model(None, dtype, shape=shape)
         pre_s = run_prefill(model, cfg, args.prefill_tokens)
@@ -410,9 +434,9 @@ def main() -> int:
     ap.add_argument("--top-p", type=float, default=1.0, help="--only serve: ... and this top-p (1: none)")
     ap.add_argument("--gather-ms", type=float, default=0.0,
                     help="--only chat: the scheduler waits this long before it admits those who came while others decode")
-    ap.add_argument("--sizes", default="1k,2k,4k", help="--only mamenex: which of the sizes " + ", ".join(MAMENEX_SIZES))
-    ap.add_argument("--kernels", action="store_true", help="--only mamenex: add the per-kernel tables (time, part of the roofline)")
-    ap.add_argument("--only", choices=["decode", "prefill", "serve", "chat", "gemm", "peaks", "mamenex"], default=None,
+    ap.add_argument("--sizes", default="1k,2k,4k", help="--only mamenex, --only nagezen: which of the sizes " + ", ".join(MAMENEX_SIZES))
+    ap.add_argument("--kernels", action="store_true", help="--only mamenex, --only nagezen: add the per-kernel tables (time, part of the roofline)")
+    ap.add_argument("--only", choices=["decode", "prefill", "serve", "chat", "gemm", "peaks", "mamenex", "nagezen"], default=None,
                     help="run one part only and print its own short line (for profiling); peaks: what a kernel that only "
                          "reads, and one of nothing but matrix-core instructions, reach on this device")
     ap.add_argument("--mnk", default="2048,11264,2048",
@@ -432,6 +456,10 @@ def main() -> int:
     if args.only == "mamenex":
         for size in args.sizes.split(","):
             print(json.dumps(run_mamenex(size, args)), flush=True)
+        return 0
+    if args.only == "nagezen":
+        for size in args.sizes.split(","):
+            print(json.dumps(run_mamenex(size, args, "nagezen", ("nagezen", "mamenex"), NAGEZEN_SIZES)), flush=True)
         return 0
     from bare_cuda_4gib_amd.csrc.peaks import measured_peaks
     measured = measured_peaks()
