@@ -325,10 +325,11 @@ int bc4g_decay_scan(const void* q, int q_dtype, long q_row, float q_scale, const
 // Attention with one or two score maps per query head over the same values (attention_maps.hip): q float32
 // [T, heads, maps, dim]; keys [page, kv_head * maps + map, token, dim], values [page, kv_head, token, vdim]; a row at p
 // sees j <= p with p - j < window or j < keep_first (window 0: all).  o = a1 - lambda a2 (one map: a1), with normalize
-// divided by sqrt(mean(o^2) + eps), times factor, times act(gate) (1: silu, 2: sigmoid; gate null: none).
+// divided by sqrt(mean(o^2) + eps), times factor, times act(gate) (1: silu, 2: sigmoid; gate null: none).  waves (1 to 8):
+// how many waves cut one row's keys among them.
 int bc4g_attention_maps(const float* q, long q_row, const void* k_cache, const void* v_cache, int cache_dtype,
                         const int32_t* block_table, int table_stride, const int32_t* row_seq, const int32_t* positions,
                         float lambda, int normalize, float eps, float factor, const void* gate, int gate_dtype, long gate_row,
                         int gate_act, void* out, int out_dtype, int n_rows, int n_heads, int n_kv_heads, int maps, int dim,
-                        int vdim, int page_tokens, int window, int keep_first, float scale, void* stream);
+                        int vdim, int page_tokens, int window, int keep_first, float scale, int waves, void* stream);
 }

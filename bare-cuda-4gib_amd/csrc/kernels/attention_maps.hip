@@ -4,9 +4,11 @@
 // scaled and gated.  Plain float arithmetic on float or bfloat16 caches: scores, weights and sums are float32.
 //
 // A row at position p sees key j if j <= p and (window == 0 or p - j < window or j < keep_first); kept keys keep their
-// own positions (they were rotated when they were written).  One wave per (row, query head): the visible keys are
-// walked in tiles of 64 in ascending order -- the kept first keys, then the window -- with a running maximum and sum per
-// map (lane = key for the scores, lane = value dimension for the sums, a tile's values read once for both maps).
+// own positions (they were rotated when they were written).  One workgroup per (row, query head): the visible keys --
+// the kept first keys, then the window -- are walked in tiles of 64, the workgroup's waves taking the tiles in turn, each
+// with a running maximum and sum per map (lane = key for the scores, lane = value dimension for the sums, a tile's
+// values read once for both maps); the waves' parts are merged in wave order.  How many waves share a row is the
+// caller's choice (few rows over long contexts: many); it changes the order of the sums and nothing else.
 // Pages that hold no visible key are never touched.
 //
 // Caches: keys [page, kv_head * maps + map, token, dim], values [page, kv_head, token, vdim].
@@ -21,7 +23,6 @@ namespace {
 
 constexpr int kMaxDim = 256;     // of a map's queries and keys
 constexpr int kMaxVdim = 256;    // of a head's values
-constexpr int kPerLane = kMaxVdim / kWave;
 
 __device__ inline float4 load_four(const float* p) { return *reinterpret_cast<const float4*>(p); }
 __device__ inline float4 load_four(const bf16_t* p) {
@@ -35,95 +36,150 @@ __device__ inline float gate_of(const void* gate, int dtype, long idx, int act) 
   return act == 1 ? z / (1.0f + expf(-z)) : 1.0f / (1.0f + expf(-z));
 }
 
-template <typename T, int MAPS>
-__global__ __launch_bounds__(kWave) void attention_maps_kernel(
+__device__ inline void wave_sync() {      // LDS written by this wave's lanes is read by its other lanes
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+constexpr int kMaxWaves = 8;     // waves of a workgroup that cut one row's keys among them
+constexpr int kAhead = 8;        // keys whose values a lane asks for together
+
+// A workgroup is one (row, query head); its NW waves take the tiles of 64 visible keys in turn (wave w the tiles w,
+// w + NW, ...), each with a running maximum and sum per map, and the waves' parts are merged in wave order at the end.
+template <typename T, int MAPS, int kNW, int VPL>      // kNW: the most waves a workgroup may have (it sizes the waves'
+                                                        // LDS); VPL: value dimensions a lane holds (vdim <= 64 VPL)
+__global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
     const float* __restrict__ q, long q_row, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seq,
     const int32_t* __restrict__ positions, float lambda, int normalize, float eps, float factor,
     const void* __restrict__ gate, int gate_dtype, long gate_row, int gate_act, void* __restrict__ out, int out_dtype,
     int n_heads, int n_kv_heads, int dim, int vdim, int page_tokens, int window, int keep_first, float scale) {
-  __shared__ float q_s[MAPS][kMaxDim];
-  __shared__ float p_s[MAPS][kWave];
-  const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  __shared__ __align__(16) float q_s[MAPS][kMaxDim];
+  __shared__ float p_s[kNW][MAPS][kWave];
+  __shared__ long v_at[kNW][kWave];           // where every key of the wave's tile has its values
+  __shared__ float part_acc[kNW > 1 ? kNW : 1][MAPS][kNW > 1 ? kMaxVdim : 1];
+  __shared__ float part_ml[kNW][MAPS][2];
+  const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int n_waves = blockDim.x / kWave;
   const int kvh = head / (n_heads / n_kv_heads);
   const int pos = positions[row];
   const int32_t* table = block_table + static_cast<long>(row_seq[row]) * table_stride;
-  for (int m = 0; m < MAPS; ++m)
-    for (int c = lane; c < dim; c += kWave) q_s[m][c] = q[row * q_row + (static_cast<long>(head) * MAPS + m) * dim + c];
+  for (int m = 0; m < MAPS; ++m)      // (zeros beyond dim: the products below run in whole batches)
+    for (int c = threadIdx.x; c < kMaxDim; c += blockDim.x)
+      q_s[m][c] = c < dim ? q[row * q_row + (static_cast<long>(head) * MAPS + m) * dim + c] : 0.f;
   __syncthreads();
 
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int kept = window > 0 ? (keep_first < first ? keep_first : first) : 0;      // kept keys before the window
   const int total = kept + (pos - first + 1);
   const bool by_four = dim % 4 == 0 && reinterpret_cast<uintptr_t>(k_cache) % (4 * sizeof(T)) == 0;
-  float mx[MAPS], sum[MAPS], acc[MAPS][kPerLane];
+  float mx[MAPS], sum[MAPS], acc[MAPS][VPL];
 #pragma unroll
   for (int m = 0; m < MAPS; ++m) {
     mx[m] = -INFINITY, sum[m] = 0.f;
 #pragma unroll
-    for (int i = 0; i < kPerLane; ++i) acc[m][i] = 0.f;
+    for (int i = 0; i < VPL; ++i) acc[m][i] = 0.f;
   }
-  for (int v0 = 0; v0 < total; v0 += kWave) {
-    const int vi = v0 + lane;
-    const bool seen = vi < total;
+  int vcol[VPL];                        // this lane's value dimensions (clamped: what lies beyond vdim is dropped at the end)
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) vcol[i] = lane + i * kWave < vdim ? lane + i * kWave : vdim - 1;
+  // Nothing in a tile's walk is under a condition: lanes without a key compute on the tile's first key and are dropped
+  // by selects, so that loads and LDS reads go out in batches.
+  for (int v0 = wave * kWave; v0 < total; v0 += n_waves * kWave) {
+    const bool seen = v0 + lane < total;
+    const int vi = seen ? v0 + lane : v0;
     const int j = vi < kept ? vi : first + (vi - kept);
-    const long page = seen ? table[j / page_tokens] : 0;
+    const long page = table[j / page_tokens];
     const int off = j % page_tokens;
+    v_at[wave][lane] = ((page * n_kv_heads + kvh) * page_tokens + off) * vdim;
 #pragma unroll
     for (int m = 0; m < MAPS; ++m) {
       float dot = 0.f;
-      if (seen) {
-        const T* kp = k_cache + ((page * (n_kv_heads * MAPS) + kvh * MAPS + m) * page_tokens + off) * dim;
-        if (by_four) {
-          for (int c = 0; c < dim; c += 4) {
-            const float4 kk = load_four(kp + c);
-            dot = fmaf(q_s[m][c], kk.x, dot), dot = fmaf(q_s[m][c + 1], kk.y, dot);
-            dot = fmaf(q_s[m][c + 2], kk.z, dot), dot = fmaf(q_s[m][c + 3], kk.w, dot);
+      const T* kp = k_cache + ((page * (n_kv_heads * MAPS) + kvh * MAPS + m) * page_tokens + off) * dim;
+      if (by_four) {
+        for (int c0 = 0; c0 < dim; c0 += 32) {            // eight loads asked for together, then their products in order
+          float4 kk[8];
+#pragma unroll
+          for (int b = 0; b < 8; ++b) kk[b] = load_four(kp + (c0 + 4 * b < dim ? c0 + 4 * b : dim - 4));
+#pragma unroll
+          for (int b = 0; b < 8; ++b) {                    // (q is zero beyond dim)
+            const float4 qq = *reinterpret_cast<const float4*>(&q_s[m][c0 + 4 * b]);
+            dot = fmaf(qq.x, kk[b].x, dot), dot = fmaf(qq.y, kk[b].y, dot);
+            dot = fmaf(qq.z, kk[b].z, dot), dot = fmaf(qq.w, kk[b].w, dot);
           }
-        } else {
-          for (int c = 0; c < dim; ++c) dot = fmaf(q_s[m][c], to_float(kp[c]), dot);
         }
+      } else {
+        for (int c = 0; c < dim; ++c) dot = fmaf(q_s[m][c], to_float(kp[c]), dot);
       }
       const float sc = seen ? dot * scale : -INFINITY;
       const float m_new = fmaxf(mx[m], wave_max(sc));       // finite: the tile's first key is visible
       const float p = seen ? expf(sc - m_new) : 0.f;
-      const float alpha = expf(mx[m] - m_new);               // 0 on the first tile
+      const float alpha = expf(mx[m] - m_new);               // 0 on the wave's first tile
       sum[m] = sum[m] * alpha + wave_sum(p);
       mx[m] = m_new;
-      p_s[m][lane] = p;
+      p_s[wave][m][lane] = p;
 #pragma unroll
-      for (int i = 0; i < kPerLane; ++i) acc[m][i] *= alpha;
+      for (int i = 0; i < VPL; ++i) acc[m][i] *= alpha;
     }
-    __syncthreads();
+    wave_sync();
     const int n_here = total - v0 < kWave ? total - v0 : kWave;
-    for (int jj = 0; jj < n_here; ++jj) {
-      const int vj = v0 + jj;
-      const int jk = vj < kept ? vj : first + (vj - kept);
-      const long pg = table[jk / page_tokens];
-      const T* vrow = v_cache + ((pg * n_kv_heads + kvh) * page_tokens + jk % page_tokens) * vdim;
+    for (int j0 = 0; j0 < n_here; j0 += kAhead) {          // lane = value dimension; kAhead keys' values asked for together
+      float vv[kAhead][VPL];                               // (keys beyond the tile's last weigh zero and read the first key's values)
 #pragma unroll
-      for (int i = 0; i < kPerLane; ++i) {
-        const int c = lane + i * kWave;
-        if (c < vdim) {
-          const float vv = to_float(vrow[c]);
+      for (int b = 0; b < kAhead; ++b) {
+        const T* vrow = v_cache + v_at[wave][j0 + b];
 #pragma unroll
-          for (int m = 0; m < MAPS; ++m) acc[m][i] = fmaf(p_s[m][jj], vv, acc[m][i]);
+        for (int i = 0; i < VPL; ++i) vv[b][i] = to_float(vrow[vcol[i]]);
+      }
+#pragma unroll
+      for (int b = 0; b < kAhead; ++b) {
+#pragma unroll
+        for (int m = 0; m < MAPS; ++m) {
+          const float p = p_s[wave][m][j0 + b];
+#pragma unroll
+          for (int i = 0; i < VPL; ++i) acc[m][i] = fmaf(p, vv[b][i], acc[m][i]);
         }
       }
     }
-    __syncthreads();
+    wave_sync();
   }
-  float o[kPerLane];
+  if (kNW > 1 && n_waves > 1) {                          // the waves' parts, merged in wave order
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+      if (lane == 0) part_ml[wave][m][0] = mx[m], part_ml[wave][m][1] = sum[m];
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) part_acc[wave][m][lane + i * kWave] = acc[m][i];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+      float top = -INFINITY;
+      for (int w = 0; w < n_waves; ++w) top = fmaxf(top, part_ml[w][m][0]);
+      sum[m] = 0.f;
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) acc[m][i] = 0.f;
+      for (int w = 0; w < n_waves; ++w) {
+        const float f = expf(part_ml[w][m][0] - top);    // 0 for a wave that had no tile
+        sum[m] = fmaf(part_ml[w][m][1], f, sum[m]);
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) acc[m][i] = fmaf(part_acc[w][m][lane + i * kWave], f, acc[m][i]);
+      }
+    }
+  }
+  float o[VPL];
   float ss = 0.f;
 #pragma unroll
-  for (int i = 0; i < kPerLane; ++i) {
+  for (int i = 0; i < VPL; ++i) {
     o[i] = acc[0][i] / sum[0];
     if (MAPS == 2) o[i] -= lambda * (acc[MAPS - 1][i] / sum[MAPS - 1]);
-    ss = fmaf(o[i], o[i], ss);          // (lanes beyond vdim hold zeros)
+    if (lane + i * kWave >= vdim) o[i] = 0.f;        // (a lane beyond vdim walked a clamped column)
+    ss = fmaf(o[i], o[i], ss);
   }
   const float mult = normalize ? factor / sqrtf(wave_sum(ss) / static_cast<float>(vdim) + eps) : factor;
 #pragma unroll
-  for (int i = 0; i < kPerLane; ++i) {
+  for (int i = 0; i < VPL; ++i) {
     const int c = lane + i * kWave;
     if (c >= vdim) break;
     float r = o[i] * mult;
@@ -144,7 +200,8 @@ extern "C" int bc4g_attention_maps(const float* q, long q_row, const void* k_cac
                                    const int32_t* positions, float lambda, int normalize, float eps, float factor,
                                    const void* gate, int gate_dtype, long gate_row, int gate_act, void* out, int out_dtype,
                                    int n_rows, int n_heads, int n_kv_heads, int maps, int dim, int vdim, int page_tokens,
-                                   int window, int keep_first, float scale, void* stream) {
+                                   int window, int keep_first, float scale, int waves, void* stream) {
+  BC4G_REQUIRE(waves >= 1 && waves <= kMaxWaves, "attention_maps: %d waves a row (1 to %d)", waves, kMaxWaves);
   BC4G_REQUIRE(n_rows >= 0 && n_heads > 0 && n_heads <= 65535 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                "attention_maps: bad sizes T=%d heads=%d/%d", n_rows, n_heads, n_kv_heads);
   BC4G_REQUIRE((maps == 1 || maps == 2) && dim > 0 && dim <= kMaxDim && vdim > 0 && vdim <= kMaxVdim,
@@ -161,7 +218,11 @@ extern "C" int bc4g_attention_maps(const float* q, long q_row, const void* k_cac
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(n_rows, n_heads);
 #define BC4G_MAPS(T, M)                                                                                                   \
-  attention_maps_kernel<T, M><<<grid, kWave, 0, s>>>(q, q_row, static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), \
+  do { if (waves == 1) BC4G_MAPS_V(T, M, 1); else BC4G_MAPS_V(T, M, kMaxWaves); } while (0)
+#define BC4G_MAPS_V(T, M, W)                                                                                              \
+  do { if (vdim <= kWave) BC4G_MAPS_W(T, M, W, 1); else if (vdim <= 2 * kWave) BC4G_MAPS_W(T, M, W, 2); else BC4G_MAPS_W(T, M, W, 4); } while (0)
+#define BC4G_MAPS_W(T, M, W, V)                                                                                           \
+  attention_maps_kernel<T, M, W, V><<<grid, waves * kWave, 0, s>>>(q, q_row, static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), \
                                                      block_table, table_stride, row_seq, positions, lambda, normalize, eps, \
                                                      factor, gate, gate_dtype, gate_row, gate_act, out, out_dtype, n_heads,  \
                                                      n_kv_heads, dim, vdim, page_tokens, window, keep_first, scale)
@@ -173,5 +234,7 @@ extern "C" int bc4g_attention_maps(const float* q, long q_row, const void* k_cac
     return fail("attention_maps: unknown dtype %d", cache_dtype);
   }
 #undef BC4G_MAPS
+#undef BC4G_MAPS_W
+#undef BC4G_MAPS_V
   return check_launch("attention_maps");
 }

@@ -171,16 +171,38 @@ __global__ __launch_bounds__(kWave) void decay_scan_kernel(const ScanArgs a) {
   for (long r0 = lo; r0 < hi; r0 += kStage) {
     const int nr = static_cast<int>(hi - r0 < kStage ? hi - r0 : kStage);
     __syncthreads();
-    for (int idx = lane; idx < nr * dim; idx += kWave) {
-      const int r = idx / dim, d = idx - r * dim;
-      const long at = static_cast<long>(head) * dim + d;
-      k_s[r][d] = load_any(a.k, a.k_dtype, (r0 + r) * a.k_row + at);
-      if (kPass) q_s[r][d] = load_any(a.q, a.q_dtype, (r0 + r) * a.q_row + at) * a.q_scale;
-      if (kPerChannel) {
-        const float zz = load_any(a.z, a.z_dtype, (r0 + r) * a.z_row + at) + (a.z_bias ? a.z_bias[at] : 0.f);
-        a_s[r][d] = expf(log_sigmoid(zz) * a.inv_tau);
+    // Eight elements a lane asked for together (a loop of single loads would wait for each in turn).  The rows lie in
+    // LDS KD wide: beyond dim the keys and queries are zero and the decays one, so that the walk below has no condition
+    // in it and its LDS reads go out in batches.
+    for (int idx0 = lane; idx0 < nr * KD; idx0 += kWave * 8) {
+      float kk[8], qq[8], zz[8];
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        const int idx = idx0 + b * kWave;
+        const int r = idx / KD, d = idx % KD;
+        const bool ok = r < nr && d < dim;
+        const long at = static_cast<long>(head) * dim + (ok ? d : 0);
+        const long row = r0 + (ok ? r : 0);
+        kk[b] = load_any(a.k, a.k_dtype, row * a.k_row + at);
+        qq[b] = kPass ? load_any(a.q, a.q_dtype, row * a.q_row + at) : 0.f;
+        zz[b] = kPerChannel ? load_any(a.z, a.z_dtype, row * a.z_row + at) + (a.z_bias ? a.z_bias[at] : 0.f) : 0.f;
+      }
+#pragma unroll
+      for (int b = 0; b < 8; ++b) {
+        const int idx = idx0 + b * kWave;
+        const int r = idx / KD, d = idx % KD;
+        if (r < nr) {
+          const bool ok = d < dim;
+          k_s[r][d] = ok ? kk[b] : 0.f;
+          if (kPass) q_s[r][d] = ok ? qq[b] * a.q_scale : 0.f;
+          if (kPerChannel) a_s[r][d] = ok ? expf(log_sigmoid(zz[b]) * a.inv_tau) : 1.0f;
+        }
       }
     }
+    float vv[kStage];                  // this thread's column of the stage's values, asked for together
+#pragma unroll
+    for (int r = 0; r < kStage; ++r)
+      vv[r] = (live && r < nr) ? load_any(a.v, a.v_dtype, (r0 + r) * a.v_row + static_cast<long>(head) * vdim + col) : 0.f;
     __syncthreads();
     if (kPass == 0 && blockIdx.x == 0) {
 #pragma unroll
@@ -190,15 +212,14 @@ __global__ __launch_bounds__(kWave) void decay_scan_kernel(const ScanArgs a) {
           for (int r = 0; r < nr; ++r) prod[i] *= kPerChannel ? a_s[r][d] : decay;
       }
     }
-    for (int r = 0; r < nr; ++r) {
-      const float vv = live ? load_any(a.v, a.v_dtype, (r0 + r) * a.v_row + static_cast<long>(head) * vdim + col) : 0.f;
+#pragma unroll
+    for (int r = 0; r < kStage; ++r) {
+      if (r >= nr) break;
       float o = 0.f;
 #pragma unroll
       for (int d = 0; d < KD; ++d) {
-        if (d < dim) {
-          S[d] = fmaf(kPerChannel ? a_s[r][d] : decay, S[d], k_s[r][d] * vv);
-          if (kPass) o = fmaf(S[d], q_s[r][d], o);
-        }
+        S[d] = fmaf(kPerChannel ? a_s[r][d] : decay, S[d], k_s[r][d] * vv[r]);
+        if (kPass) o = fmaf(S[d], q_s[r][d], o);
       }
       if (kPass && live) a.out[((r0 + r) * a.heads + head) * vdim + col] = o;
     }
@@ -238,12 +259,23 @@ __global__ void decay_scan_between_kernel(float* __restrict__ state, float* __re
   const int d = static_cast<int>(e / vdim);
   float* slot = state + (static_cast<long>(seq_slots[s]) * heads + head) * per_state + e;
   float st = *slot;
-  for (int c = 0; c < n_chunks; ++c) {
-    const long id = chunk_base[s] + c;
-    float* sum = chunk_state + (id * heads + head) * per_state + e;
-    const float add = *sum;
-    *sum = st;
-    st = fmaf(chunk_decay[(id * heads + head) * dim + d], st, add);
+  const long id0 = chunk_base[s];
+  for (int c0 = 0; c0 < n_chunks; c0 += 8) {          // (eight chunks' numbers asked for together)
+    float add[8], dec[8];
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      const bool ok = c0 + b < n_chunks;
+      const long id = id0 + (ok ? c0 + b : 0);
+      add[b] = ok ? chunk_state[(id * heads + head) * per_state + e] : 0.f;
+      dec[b] = ok ? chunk_decay[(id * heads + head) * dim + d] : 1.f;
+    }
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      if (c0 + b < n_chunks) {
+        chunk_state[((id0 + c0 + b) * heads + head) * per_state + e] = st;
+        st = fmaf(dec[b], st, add[b]);
+      }
+    }
   }
   *slot = st;
 }
@@ -339,7 +371,8 @@ extern "C" int bc4g_decay_scan(const void* q, int q_dtype, long q_row, float q_s
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(ceil_div(vdim, kWave), most_chunks, n_seqs * heads);
   const bool per_channel = z != nullptr;
-  if (dim <= 32) launch_scan<32>(a, per_channel, chunked, grid, s);
+  if (dim <= 16) launch_scan<16>(a, per_channel, chunked, grid, s);
+  else if (dim <= 32) launch_scan<32>(a, per_channel, chunked, grid, s);
   else if (dim <= 64) launch_scan<64>(a, per_channel, chunked, grid, s);
   else if (dim <= 128) launch_scan<128>(a, per_channel, chunked, grid, s);
   else launch_scan<256>(a, per_channel, chunked, grid, s);

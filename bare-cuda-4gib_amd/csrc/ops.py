@@ -1485,6 +1485,7 @@ HEADS_MAX_DIM = 256         # elements of a head that heads_prepare, heads_finis
 DECAY_SCAN_CHUNK = 64       # rows of a request that one workgroup of the scan walks
 
 ACT_NONE, ACT_SILU, ACT_SIGMOID = 0, 1, 2
+ATTENTION_MAPS_FULL = 4096   # (row, head) pairs from which on one wave walks a row's keys alone
 
 
 def _part_of_rows(what: str, name: str, t: torch.Tensor, width: int) -> int:
@@ -1625,11 +1626,13 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.T
 def attention_maps(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor, ctx, out_dtype: torch.dtype,
                    n_heads: int, n_kv_heads: int, maps: int, dim: int, vdim: int, window: int, keep_first: int, scale: float, *,
                    lam: float = 0.0, normalize: bool = False, eps: float = 0.0, factor: float = 1.0,
-                   gate: Optional[torch.Tensor] = None, act: int = ACT_SIGMOID) -> torch.Tensor:
+                   gate: Optional[torch.Tensor] = None, act: int = ACT_SIGMOID, waves: int = 0) -> torch.Tensor:
     """Softmax attention with ``maps`` (1 or 2) score maps per query head over the same values: q float32
     [T, n_heads, maps, dim]; keys [pages, n_kv_heads * maps, page_tokens, dim], values [pages, n_kv_heads, page_tokens, vdim].
     A row at position p sees key j <= p if p - j < window or j < keep_first (window 0: every key).  o = a1 - lam a2,
-    with ``normalize`` divided by sqrt(mean(o^2) + eps) over the head, times ``factor`` and act(gate); [T, n_heads * vdim]."""
+    with ``normalize`` divided by sqrt(mean(o^2) + eps) over the head, times ``factor`` and act(gate); [T, n_heads * vdim].
+    ``waves``: how many waves cut one row's keys among them (0: chosen here -- one where the rows fill the GPU, up to
+    eight where few rows walk long contexts)."""
     _dev("attention_maps", q, k_cache, v_cache, block_table)
     t = q.shape[0]
     if q.dtype != torch.float32 or tuple(q.shape) != (t, n_heads, maps, dim):
@@ -1659,9 +1662,13 @@ def attention_maps(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
                 keys += cached + new
         return (2.0 * pairs * n_heads * maps * (dim + vdim),
                 keys * n_kv_heads * (maps * dim + vdim) * k_cache.element_size() + t * n_heads * (4 * maps * dim + vdim * out.element_size()))
+    if waves <= 0:
+        reach = ctx.max_kv_len if window <= 0 else min(ctx.max_kv_len, window + keep_first)
+        tiles = max(1, -(-reach // 64))
+        waves = 1 if t * n_heads >= ATTENTION_MAPS_FULL else min(8, tiles)
     library.call("bc4g_attention_maps", _ptr(q), n_heads * maps * dim, _ptr(k_cache), _ptr(v_cache), _code(k_cache, "attention_maps"),
                  _ptr(block_table), block_table.stride(0), _ptr(ctx.row_seq), _ptr(ctx.positions), float(lam), 1 if normalize else 0,
                  float(eps), float(factor), _ptr(gate), _code(gate, "attention_maps") if gate is not None else F32, gate_row, int(act),
                  _ptr(out), _code(out, "attention_maps"), t, n_heads, n_kv_heads, maps, dim, vdim, page_tokens, int(window),
-                 int(keep_first), float(scale), _stream(), cost=cost)
+                 int(keep_first), float(scale), int(waves), _stream(), cost=cost)
     return out
