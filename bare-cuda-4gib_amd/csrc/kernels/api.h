@@ -313,7 +313,7 @@ int bc4g_heads_finish(const float* o, const float* w, float eps, float factor, c
                       int act, void* out, int out_dtype, int n_rows, int heads, int vdim, void* stream);
 // S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T (q_t q_scale) along every request's rows, from state
 // [slots, heads, dim, vdim] (float32) and back into it; out float32 [T, heads, vdim].  a_t = head_decay[head], or with
-// gate logits z [T, heads, dim]: sigmoid(z + z_bias)^inv_tau.  Requests that bring more than 64 rows are walked in
+// gate logits z [T, heads, dim]: sigmoid(z + z_bias)^inv_tau.  Requests that bring more than 32 rows are walked in
 // chunks: chunk_state [chunks, heads, dim, vdim], chunk_decay [chunks, heads, dim] (float32 scratch) and chunk_base [S],
 // the first chunk of every request among all chunks of requests that have two or more.  dim at most 256.
 int bc4g_decay_scan(const void* q, int q_dtype, long q_row, float q_scale, const void* k, int k_dtype, long k_row,

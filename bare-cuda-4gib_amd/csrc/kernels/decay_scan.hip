@@ -10,7 +10,7 @@
 //             a dense tensor or into the pages of a cache.
 //   finish    per (row, head): o / rms(o) (* weight) * factor * act(gate).
 //
-// The scan walks a request's rows in chunks of 64, each chunk by workgroups of its own (a thread keeps one column of
+// The scan walks a request's rows in chunks of 32, each chunk by workgroups of its own (a thread keeps one column of
 // the state, dim numbers, in registers): first every chunk from a zero state (what it adds, and the product of its
 // decays), then the states between the chunks in a short sequential pass, then every chunk again from its true
 // state, writing outputs.  A request that brings at most one chunk (a decode step) takes the last pass alone, from
@@ -23,7 +23,7 @@
 namespace bc4g {
 namespace {
 
-constexpr int kChunk = 64;       // rows of a request that one workgroup walks
+constexpr int kChunk = 32;       // rows of a request that one workgroup walks
 constexpr int kStage = 16;       // rows whose q, k and decays lie in LDS at a time
 constexpr int kMaxHead = 256;    // elements of a head that prepare and finish take
 

@@ -1482,7 +1482,7 @@ def clamped_glu(gu: torch.Tensor, limit: float, slope: float) -> torch.Tensor:
 # ---- heads: rotation tables, preparation, finishing; linear attention with a decayed state; attention with two maps -----
 
 HEADS_MAX_DIM = 256         # elements of a head that heads_prepare, heads_finish, decay_scan and attention_maps take
-DECAY_SCAN_CHUNK = 64       # rows of a request that one workgroup of the scan walks
+DECAY_SCAN_CHUNK = 32       # rows of a request that one workgroup of the scan walks
 
 ACT_NONE, ACT_SILU, ACT_SIGMOID = 0, 1, 2
 ATTENTION_MAPS_FULL = 4096   # (row, head) pairs from which on one wave walks a row's keys alone

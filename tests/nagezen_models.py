@@ -55,7 +55,7 @@ CONFIGS: Dict[str, dict] = {
         gla(5, 5, 70, tau=9.0, rank=3, ff=96),
         attention(6, 1, 24, 130, window=50, keep_first=7, dims=24, scale=0.3, diff=0.55),
         retention(2, 40, 24, [0.5, 0.999], ff=72, limit=5.0)]),
-    "C": dict(architecture="Nagezen", vocab=77, width=40, streams=5, logit_scale=0.25, norm=dict(eps=1e-3), layers=[
+    "C": dict(architecture="Nagezen", vocab=77, width=42, streams=5, logit_scale=0.25, norm=dict(eps=1e-3), layers=[
         attention(2, 2, 6, 9, dims=2, base=30.0, diff=0.1, ff=44),                                   # no window: every key
         retention(1, 72, 7, [0.98], dims=72, base=1000.0),
         attention(5, 1, 7, 5, window=6, keep_first=10, dims=6, scaling=dict(factor=2.0, original=16, fast=4.0, slow=1.0), diff=0.8),
