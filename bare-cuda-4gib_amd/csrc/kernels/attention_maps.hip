@@ -47,8 +47,11 @@ constexpr int kAhead = 8;        // keys whose values a lane asks for together
 
 // A workgroup is one (row, query head); its NW waves take the tiles of 64 visible keys in turn (wave w the tiles w,
 // w + NW, ...), each with a running maximum and sum per map, and the waves' parts are merged in wave order at the end.
-template <typename T, int MAPS, int kNW, int VPL>      // kNW: the most waves a workgroup may have (it sizes the waves'
-                                                        // LDS); VPL: value dimensions a lane holds (vdim <= 64 VPL)
+// kNW: the most waves a workgroup may have (it sizes the waves' LDS); VPL: value dimensions a lane holds (vdim <= 64 VPL);
+// E4: for the scores, eight lanes share a key and each takes 4 E4 of its dimensions (dim <= 32 E4), so that a load's lanes
+// read eight keys' rows end to end -- with a key to a lane every load touched 64 cache lines, and the kernel was as long as
+// the CU's one path to memory took to serve them.
+template <typename T, int MAPS, int kNW, int VPL, int E4>
 __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
     const float* __restrict__ q, long q_row, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seq,
@@ -58,6 +61,8 @@ __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
   __shared__ __align__(16) float q_s[MAPS][kMaxDim];
   __shared__ float p_s[kNW][MAPS][kWave];
   __shared__ long v_at[kNW][kWave];           // where every key of the wave's tile has its values
+  __shared__ long k_at[kNW][kWave];           // ... and its first map's dimensions
+  __shared__ float s_s[kNW][MAPS][kWave];     // the tile's scores on their way from (key, piece) lanes to lane = key
   __shared__ float part_acc[kNW > 1 ? kNW : 1][MAPS][kNW > 1 ? kMaxVdim : 1];
   __shared__ float part_ml[kNW][MAPS][2];
   const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -84,6 +89,16 @@ __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
   int vcol[VPL];                        // this lane's value dimensions (clamped: what lies beyond vdim is dropped at the end)
 #pragma unroll
   for (int i = 0; i < VPL; ++i) vcol[i] = lane + i * kWave < vdim ? lane + i * kWave : vdim - 1;
+  const int sub = lane / 8, piece = lane % 8;          // for the scores: which of a load's eight keys, which piece of its dimensions
+  float4 q_r[MAPS][E4];                                 // this lane's piece of the queries (zero beyond dim)
+  int k_col[E4];                                        // ... and where it lies in a key's row (clamped)
+#pragma unroll
+  for (int e = 0; e < E4; ++e) {
+    const int c = piece * 4 * E4 + 4 * e;
+    k_col[e] = c + 4 <= dim ? c : (dim >= 4 ? dim - 4 : 0);
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) q_r[m][e] = *reinterpret_cast<const float4*>(&q_s[m][c]);
+  }
   // Nothing in a tile's walk is under a condition: lanes without a key compute on the tile's first key and are dropped
   // by selects, so that loads and LDS reads go out in batches.
   for (int v0 = wave * kWave; v0 < total; v0 += n_waves * kWave) {
@@ -93,23 +108,43 @@ __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
     const long page = table[j / page_tokens];
     const int off = j % page_tokens;
     v_at[wave][lane] = ((page * n_kv_heads + kvh) * page_tokens + off) * vdim;
+    if (by_four) {
+      k_at[wave][lane] = ((page * (n_kv_heads * MAPS) + kvh * MAPS) * page_tokens + off) * dim;
+      wave_sync();
+#pragma unroll
+      for (int it = 0; it < 8; it += 2) {                  // sixteen keys' pieces asked for together
+        float4 kk[2][MAPS][E4];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const T* kp = k_cache + k_at[wave][8 * (it + u) + sub];
+#pragma unroll
+          for (int m = 0; m < MAPS; ++m)
+#pragma unroll
+            for (int e = 0; e < E4; ++e) kk[u][m][e] = load_four(kp + static_cast<long>(m) * page_tokens * dim + k_col[e]);
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int m = 0; m < MAPS; ++m) {
+            float part = 0.f;
+#pragma unroll
+            for (int e = 0; e < E4; ++e) {
+              part = fmaf(q_r[m][e].x, kk[u][m][e].x, part), part = fmaf(q_r[m][e].y, kk[u][m][e].y, part);
+              part = fmaf(q_r[m][e].z, kk[u][m][e].z, part), part = fmaf(q_r[m][e].w, kk[u][m][e].w, part);
+            }
+            part += __shfl_xor(part, 1, kWave), part += __shfl_xor(part, 2, kWave), part += __shfl_xor(part, 4, kWave);
+            if (piece == 0) s_s[wave][m][8 * (it + u) + sub] = part;
+          }
+      }
+      wave_sync();
+    }
 #pragma unroll
     for (int m = 0; m < MAPS; ++m) {
       float dot = 0.f;
-      const T* kp = k_cache + ((page * (n_kv_heads * MAPS) + kvh * MAPS + m) * page_tokens + off) * dim;
       if (by_four) {
-        for (int c0 = 0; c0 < dim; c0 += 32) {            // eight loads asked for together, then their products in order
-          float4 kk[8];
-#pragma unroll
-          for (int b = 0; b < 8; ++b) kk[b] = load_four(kp + (c0 + 4 * b < dim ? c0 + 4 * b : dim - 4));
-#pragma unroll
-          for (int b = 0; b < 8; ++b) {                    // (q is zero beyond dim)
-            const float4 qq = *reinterpret_cast<const float4*>(&q_s[m][c0 + 4 * b]);
-            dot = fmaf(qq.x, kk[b].x, dot), dot = fmaf(qq.y, kk[b].y, dot);
-            dot = fmaf(qq.z, kk[b].z, dot), dot = fmaf(qq.w, kk[b].w, dot);
-          }
-        }
+        dot = s_s[wave][m][lane];
       } else {
+        const T* kp = k_cache + ((page * (n_kv_heads * MAPS) + kvh * MAPS + m) * page_tokens + off) * dim;
         for (int c = 0; c < dim; ++c) dot = fmaf(q_s[m][c], to_float(kp[c]), dot);
       }
       const float sc = seen ? dot * scale : -INFINITY;
@@ -222,7 +257,9 @@ extern "C" int bc4g_attention_maps(const float* q, long q_row, const void* k_cac
 #define BC4G_MAPS_V(T, M, W)                                                                                              \
   do { if (vdim <= kWave) BC4G_MAPS_W(T, M, W, 1); else if (vdim <= 2 * kWave) BC4G_MAPS_W(T, M, W, 2); else BC4G_MAPS_W(T, M, W, 4); } while (0)
 #define BC4G_MAPS_W(T, M, W, V)                                                                                           \
-  attention_maps_kernel<T, M, W, V><<<grid, waves * kWave, 0, s>>>(q, q_row, static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), \
+  do { if (dim <= 64) BC4G_MAPS_E(T, M, W, V, 2); else BC4G_MAPS_E(T, M, W, V, 8); } while (0)
+#define BC4G_MAPS_E(T, M, W, V, E)                                                                                        \
+  attention_maps_kernel<T, M, W, V, E><<<grid, waves * kWave, 0, s>>>(q, q_row, static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), \
                                                      block_table, table_stride, row_seq, positions, lambda, normalize, eps, \
                                                      factor, gate, gate_dtype, gate_row, gate_act, out, out_dtype, n_heads,  \
                                                      n_kv_heads, dim, vdim, page_tokens, window, keep_first, scale)
@@ -236,5 +273,6 @@ extern "C" int bc4g_attention_maps(const float* q, long q_row, const void* k_cac
 #undef BC4G_MAPS
 #undef BC4G_MAPS_W
 #undef BC4G_MAPS_V
+#undef BC4G_MAPS_E
   return check_launch("attention_maps");
 }
