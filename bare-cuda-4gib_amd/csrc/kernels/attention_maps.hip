@@ -47,11 +47,14 @@ constexpr int kAhead = 8;        // keys whose values a lane asks for together
 
 // A workgroup is one (row, query head); its NW waves take the tiles of 64 visible keys in turn (wave w the tiles w,
 // w + NW, ...), each with a running maximum and sum per map, and the waves' parts are merged in wave order at the end.
-// kNW: the most waves a workgroup may have (it sizes the waves' LDS); VPL: value dimensions a lane holds (vdim <= 64 VPL);
+// kNW: the most waves a workgroup may have (it sizes the waves' LDS).  LPK: lanes that share a key for the weighted sums, each
+// with four neighbouring value dimensions (vdim <= 4 LPK; 16, 32 or 64), so that a load brings 64 / LPK keys' values in
+// pieces of four and the groups' sums are added across lanes at the end; 0: a lane holds dimensions lane, lane + 64, ...
+// one key a load (any vdim).
 // E4: for the scores, eight lanes share a key and each takes 4 E4 of its dimensions (dim <= 32 E4), so that a load's lanes
 // read eight keys' rows end to end -- with a key to a lane every load touched 64 cache lines, and the kernel was as long as
 // the CU's one path to memory took to serve them.
-template <typename T, int MAPS, int kNW, int VPL, int E4>
+template <typename T, int MAPS, int kNW, int LPK, int E4>
 __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
     const float* __restrict__ q, long q_row, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seq,
@@ -79,6 +82,9 @@ __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
   const int kept = window > 0 ? (keep_first < first ? keep_first : first) : 0;      // kept keys before the window
   const int total = kept + (pos - first + 1);
   const bool by_four = dim % 4 == 0 && reinterpret_cast<uintptr_t>(k_cache) % (4 * sizeof(T)) == 0;
+  constexpr int VPL = 4;                // value dimensions a lane holds
+  constexpr int KPI = LPK ? kWave / LPK : 1;      // keys a load of values brings
+  const int vgroup = LPK ? lane / LPK : 0;
   float mx[MAPS], sum[MAPS], acc[MAPS][VPL];
 #pragma unroll
   for (int m = 0; m < MAPS; ++m) {
@@ -86,9 +92,10 @@ __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
 #pragma unroll
     for (int i = 0; i < VPL; ++i) acc[m][i] = 0.f;
   }
-  int vcol[VPL];                        // this lane's value dimensions (clamped: what lies beyond vdim is dropped at the end)
+  int vcol[VPL];                        // this lane's value dimensions (what lies beyond vdim is dropped at the end)
 #pragma unroll
-  for (int i = 0; i < VPL; ++i) vcol[i] = lane + i * kWave < vdim ? lane + i * kWave : vdim - 1;
+  for (int i = 0; i < VPL; ++i) vcol[i] = LPK ? 4 * (lane % (LPK ? LPK : 1)) + i : lane + i * kWave;
+  const int vfrom = LPK ? (vcol[0] + 4 <= vdim ? vcol[0] : vdim - 4) : 0;      // where this lane's piece of four is read (clamped)
   const int sub = lane / 8, piece = lane % 8;          // for the scores: which of a load's eight keys, which piece of its dimensions
   float4 q_r[MAPS][E4];                                 // this lane's piece of the queries (zero beyond dim)
   int k_col[E4];                                        // ... and where it lies in a key's row (clamped)
@@ -159,19 +166,25 @@ __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
     }
     wave_sync();
     const int n_here = total - v0 < kWave ? total - v0 : kWave;
-    for (int j0 = 0; j0 < n_here; j0 += kAhead) {          // lane = value dimension; kAhead keys' values asked for together
-      float vv[kAhead][VPL];                               // (keys beyond the tile's last weigh zero and read the first key's values)
+    // (keys beyond the tile's last weigh zero and read the first key's values)
+    for (int j0 = 0; j0 < n_here; j0 += kAhead * KPI) {    // kAhead loads asked for together
+      float vv[kAhead][VPL];
 #pragma unroll
       for (int b = 0; b < kAhead; ++b) {
-        const T* vrow = v_cache + v_at[wave][j0 + b];
+        const T* vrow = v_cache + v_at[wave][j0 + b * KPI + vgroup];
+        if (LPK) {
+          const float4 four = load_four(vrow + vfrom);
+          vv[b][0] = four.x, vv[b][1] = four.y, vv[b][2] = four.z, vv[b][3] = four.w;
+        } else {
 #pragma unroll
-        for (int i = 0; i < VPL; ++i) vv[b][i] = to_float(vrow[vcol[i]]);
+          for (int i = 0; i < VPL; ++i) vv[b][i] = to_float(vrow[vcol[i] < vdim ? vcol[i] : vdim - 1]);
+        }
       }
 #pragma unroll
       for (int b = 0; b < kAhead; ++b) {
 #pragma unroll
         for (int m = 0; m < MAPS; ++m) {
-          const float p = p_s[wave][m][j0 + b];
+          const float p = p_s[wave][m][j0 + b * KPI + vgroup];
 #pragma unroll
           for (int i = 0; i < VPL; ++i) acc[m][i] = fmaf(p, vv[b][i], acc[m][i]);
         }
@@ -179,12 +192,23 @@ __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
     }
     wave_sync();
   }
+  if (LPK && LPK < kWave) {                              // the groups of lanes that took different keys: their sums together
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m)
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        if (LPK <= 16) acc[m][i] += __shfl_xor(acc[m][i], 16, kWave);
+        acc[m][i] += __shfl_xor(acc[m][i], 32, kWave);
+      }
+  }
+  const bool writer = !LPK || lane < LPK;                // (the other lanes hold copies)
   if (kNW > 1 && n_waves > 1) {                          // the waves' parts, merged in wave order
 #pragma unroll
     for (int m = 0; m < MAPS; ++m) {
       if (lane == 0) part_ml[wave][m][0] = mx[m], part_ml[wave][m][1] = sum[m];
 #pragma unroll
-      for (int i = 0; i < VPL; ++i) part_acc[wave][m][lane + i * kWave] = acc[m][i];
+      for (int i = 0; i < VPL; ++i)
+        if (writer) part_acc[wave][m][vcol[i]] = acc[m][i];
     }
     __syncthreads();
     if (wave != 0) return;
@@ -199,7 +223,7 @@ __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
         const float f = expf(part_ml[w][m][0] - top);    // 0 for a wave that had no tile
         sum[m] = fmaf(part_ml[w][m][1], f, sum[m]);
 #pragma unroll
-        for (int i = 0; i < VPL; ++i) acc[m][i] = fmaf(part_acc[w][m][lane + i * kWave], f, acc[m][i]);
+        for (int i = 0; i < VPL; ++i) acc[m][i] = fmaf(part_acc[w][m][vcol[i]], f, acc[m][i]);
       }
     }
   }
@@ -209,14 +233,14 @@ __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
   for (int i = 0; i < VPL; ++i) {
     o[i] = acc[0][i] / sum[0];
     if (MAPS == 2) o[i] -= lambda * (acc[MAPS - 1][i] / sum[MAPS - 1]);
-    if (lane + i * kWave >= vdim) o[i] = 0.f;        // (a lane beyond vdim walked a clamped column)
+    if (vcol[i] >= vdim || !writer) o[i] = 0.f;      // (a lane beyond vdim walked a clamped column; copies count once)
     ss = fmaf(o[i], o[i], ss);
   }
   const float mult = normalize ? factor / sqrtf(wave_sum(ss) / static_cast<float>(vdim) + eps) : factor;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
-    const int c = lane + i * kWave;
-    if (c >= vdim) break;
+    const int c = vcol[i];
+    if (c >= vdim || !writer) continue;
     float r = o[i] * mult;
     if (gate) r *= gate_of(gate, gate_dtype, row * gate_row + static_cast<long>(head) * vdim + c, gate_act);
     const long at = (static_cast<long>(row) * n_heads + head) * vdim + c;
@@ -252,10 +276,11 @@ extern "C" int bc4g_attention_maps(const float* q, long q_row, const void* k_cac
   if (n_rows == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(n_rows, n_heads);
+  const bool v_four = vdim % 4 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0;
 #define BC4G_MAPS(T, M)                                                                                                   \
   do { if (waves == 1) BC4G_MAPS_V(T, M, 1); else BC4G_MAPS_V(T, M, kMaxWaves); } while (0)
 #define BC4G_MAPS_V(T, M, W)                                                                                              \
-  do { if (vdim <= kWave) BC4G_MAPS_W(T, M, W, 1); else if (vdim <= 2 * kWave) BC4G_MAPS_W(T, M, W, 2); else BC4G_MAPS_W(T, M, W, 4); } while (0)
+  do { if (!v_four) BC4G_MAPS_W(T, M, W, 0); else if (vdim <= 64) BC4G_MAPS_W(T, M, W, 16); else if (vdim <= 128) BC4G_MAPS_W(T, M, W, 32); else BC4G_MAPS_W(T, M, W, 64); } while (0)
 #define BC4G_MAPS_W(T, M, W, V)                                                                                           \
   do { if (dim <= 64) BC4G_MAPS_E(T, M, W, V, 2); else BC4G_MAPS_E(T, M, W, V, 8); } while (0)
 #define BC4G_MAPS_E(T, M, W, V, E)                                                                                        \
