@@ -83,10 +83,10 @@ def nagezen_shape(width, layers, heads, kv_heads, dim, vdim, ff, streams=4, wind
     mlp = dict(kind="dense", ff=ff, limit=7.0)
     att = dict(type="attention", mlp=mlp, mixer=dict(
         heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, diff=0.5, scale=dim ** -0.5, mask=dict(size=window, keep_first=keep_first),
-        rot=dict(base=10000.0, dims=dim, scaling=dict(factor=4.0, original=2048, fast=32.0, slow=1.0))))
-    gla = dict(type="gla", mlp=mlp, mixer=dict(heads=heads, dim=dim, vdim=vdim, tau=16.0, rank=16))
+        rot=dict(base=10000.0, dims=dim, scaling=dict(factor=8.0, original=4096, fast=24.0, slow=2.0))))
+    gla = dict(type="gla", mlp=mlp, mixer=dict(heads=heads, dim=dim, vdim=vdim, tau=8.0, rank=32))
     ret = dict(type="retention", mlp=mlp, mixer=dict(heads=heads, dim=dim, vdim=vdim, rot=dict(base=10000.0, dims=dim),
-                                                     decay=[1.0 - 2.0 ** -(5 + 4 * a // heads) for a in range(heads)]))
+                                                     decay=[1.0 - 2.0 ** -(4 + 5 * a // heads) for a in range(heads)]))
     order = [att if i % 3 == 0 else (gla if i % 3 == 1 else ret) for i in range(layers)]
     return dict(architecture="Nagezen", vocab=vocab, width=width, streams=streams, logit_scale=1.0, norm=dict(eps=1e-6), layers=order)
 

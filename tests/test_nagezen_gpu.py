@@ -294,8 +294,8 @@ def test_clamped_gated_unit(dtype):
     assert float(plain.clamped_glu(torch.tensor([-9.0]), torch.tensor([0.0]), 2.5)) < -1e-6      # (no clamp below on the gate)
 
 
-@pytest.mark.parametrize("scaling", [None, dict(factor=8.0, original=64, fast=16.0, slow=2.0), dict(factor=3.0, original=4096, fast=32.0, slow=1.0)])
-@pytest.mark.parametrize("dims,base", [(2, 10.0), (8, 500.0), (48, 20000.0)])
+@pytest.mark.parametrize("scaling", [None, dict(factor=8.0, original=64, fast=16.0, slow=2.0), dict(factor=3.0, original=4096, fast=24.0, slow=1.5)])
+@pytest.mark.parametrize("dims,base", [(2, 10.0), (8, 500.0), (40, 30000.0)])
 def test_rotation_tables_far_from_the_start(scaling, dims, base):
     from bare_cuda_4gib_amd.engine.spec import PartSpec
     from bare_cuda_4gib_amd.parts import build_part
@@ -360,7 +360,7 @@ def test_heads_are_normed_and_gated(dtype, heads, vdim):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("heads,dim,vdim", [(3, 5, 12), (2, 40, 70), (1, 72, 7), (1, 130, 33), (2, 64, 128)])
+@pytest.mark.parametrize("heads,dim,vdim", [(3, 5, 12), (2, 40, 70), (1, 72, 7), (1, 130, 33), (2, 64, 128), (2, 24, 20)])
 @pytest.mark.parametrize("per_channel", [False, True])
 def test_decayed_state_over_portions(dtype, heads, dim, vdim, per_channel):
     """Two requests of unequal length in portions of 1 to 200 rows (one chunk, several chunks, chunks' edges), in state
@@ -441,7 +441,7 @@ def plain_maps(q, keys, values, pos, G, maps, scale, window, keep_first, lam):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("sizes", [(4, 2, 2, 12, 20), (3, 3, 1, 10, 70), (6, 1, 2, 44, 100), (2, 1, 2, 7, 130)])
+@pytest.mark.parametrize("sizes", [(4, 2, 2, 12, 20), (3, 3, 1, 10, 70), (6, 1, 2, 44, 100), (2, 1, 2, 7, 130), (2, 2, 2, 72, 200), (4, 1, 1, 128, 64)])
 @pytest.mark.parametrize("needle", [0, 7, 8, 63, 64, 120, 199])
 def test_attention_finds_one_key_among_hundreds(dtype, needle, sizes):
     """200 cached keys in scattered pages of 8, no window; one key, far back, at a page's border or the row's own, is
