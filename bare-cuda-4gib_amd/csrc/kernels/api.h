@@ -289,7 +289,7 @@ int bc4g_clamped_glu(const void* gu, void* out, int dtype, float limit, float sl
 // A residual stream in n copies, x [T, n, H] float32 (streams.hip).  read: out[r] = N(sum_s read[s] x[rows ? rows[r] : r, s])
 // with N(u) = (tanh(alpha u) g + b) out_scale (alpha null: out = the sum; read null: every copy counts once).  write:
 // x'[t] = sum_s mix[s, t] x[s] + write[t] y for all copies at once, and with next_out also the next reader's input
-// N(sum_t next_read[t] x'[t]).  fill: every copy = in.  At most 8 copies.
+// N(sum_t next_read[t] x'[t]).  fill: every copy = in.  At most 16 copies.
 int bc4g_streams_read(const float* x, const int32_t* rows, const float* read, const float* alpha, const float* g, const float* b,
                       float out_scale, void* out, int out_dtype, int n_rows, int n_streams, int hidden, void* stream);
 int bc4g_streams_write(float* x, const float* y, const float* mix, const float* write, const float* next_read,
@@ -303,6 +303,14 @@ int bc4g_rotary_table(const int32_t* positions, const double* freqs, double amp,
 // (null: none), rotation of the first 2 * half elements by the table (element i with element i + half), times factor;
 // into out [T, heads, dim] (rows out_row apart) or, with slot_map (slot = page * page_tokens + offset), into a cache
 // at out + page * page_stride + head * head_stride + offset * token_stride.  dim at most 256.
+// The same for up to four sections of the same rows in one launch: every field as the argument of that name below.
+struct bc4g_prepare_section {
+  const void* in; const float* bias; const float* norm_w; const float* table; void* out; const int32_t* slot_map;
+  long in_row, out_row, page_stride, head_stride, token_stride;
+  int in_dtype, out_dtype, half, page_tokens, heads, dim;
+  float eps, factor;
+};
+int bc4g_heads_prepare_many(const bc4g_prepare_section* sections, int n_sections, int n_rows, void* stream);
 int bc4g_heads_prepare(const void* in, int in_dtype, long in_row, const float* bias, const float* norm_w, float eps,
                        const float* table, int half, float factor, void* out, int out_dtype, long out_row,
                        const int32_t* slot_map, int page_tokens, long page_stride, long head_stride, long token_stride,

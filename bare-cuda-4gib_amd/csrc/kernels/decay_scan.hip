@@ -47,29 +47,39 @@ __global__ void rotary_table_kernel(const int32_t* __restrict__ positions, const
   }
 }
 
-// One wave per (row, head).
-__global__ __launch_bounds__(kWave) void heads_prepare_kernel(
-    const void* __restrict__ in, int in_dtype, long in_row, const float* __restrict__ bias, const float* __restrict__ norm_w,
-    float eps, const float* __restrict__ table, int half, float factor, void* __restrict__ out, int out_dtype, long out_row,
-    const int32_t* __restrict__ slot_map, int page_tokens, long page_stride, long head_stride, long token_stride, int dim) {
+// One wave per (row, head); the heads of up to four sections of one step's rows in one launch (the queries, keys and
+// values of an attention layer, say), each section with its own input, size, bias, norm, rotation, factor and output.
+struct PrepareSections {
+  bc4g_prepare_section s[4];
+  int n;
+};
+
+__global__ __launch_bounds__(kWave) void heads_prepare_kernel(const PrepareSections all) {
   __shared__ float vals[kMaxHead];
-  const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const int row = blockIdx.x, lane = threadIdx.x;
+  int head = blockIdx.y, which = 0;
+  while (which + 1 < all.n && head >= all.s[which].heads) head -= all.s[which].heads, ++which;
+  const bc4g_prepare_section& p = all.s[which];
+  const int dim = p.dim, half = p.half;
+  const float* bias = p.bias;
+  const float* norm_w = p.norm_w;
+  const float* table = p.table;
   float ss = 0.f;
   for (int c = lane; c < dim; c += kWave) {
-    float v = load_any(in, in_dtype, row * in_row + static_cast<long>(head) * dim + c);
+    float v = load_any(p.in, p.in_dtype, row * p.in_row + static_cast<long>(head) * dim + c);
     if (bias) v += bias[static_cast<long>(head) * dim + c];
     vals[c] = v;
     ss = fmaf(v, v, ss);
   }
   float scale = 1.0f;
-  if (norm_w) scale = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(dim) + eps);
+  if (norm_w) scale = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(dim) + p.eps);
   __syncthreads();
   long base;
-  if (slot_map) {
-    const long slot = slot_map[row];
-    base = (slot / page_tokens) * page_stride + head * head_stride + (slot % page_tokens) * token_stride;
+  if (p.slot_map) {
+    const long slot = p.slot_map[row];
+    base = (slot / p.page_tokens) * p.page_stride + head * p.head_stride + (slot % p.page_tokens) * p.token_stride;
   } else {
-    base = row * out_row + static_cast<long>(head) * dim;
+    base = row * p.out_row + static_cast<long>(head) * dim;
   }
   for (int c = lane; c < dim; c += kWave) {
     float v;
@@ -83,7 +93,7 @@ __global__ __launch_bounds__(kWave) void heads_prepare_kernel(
       v = vals[c] * scale;
       if (norm_w) v *= norm_w[c];
     }
-    store_any(out, out_dtype, base + c, v * factor);
+    store_any(p.out, p.out_dtype, base + c, v * p.factor);
   }
 }
 
@@ -313,22 +323,37 @@ extern "C" int bc4g_rotary_table(const int32_t* positions, const double* freqs, 
   return check_launch("rotary_table");
 }
 
+extern "C" int bc4g_heads_prepare_many(const bc4g_prepare_section* sections, int n_sections, int n_rows, void* stream) {
+  BC4G_REQUIRE(sections && n_sections >= 1 && n_sections <= 4 && n_rows >= 0, "heads_prepare: %d sections (1 to 4), %d rows",
+               n_sections, n_rows);
+  PrepareSections all;
+  long heads = 0;
+  for (int i = 0; i < n_sections; ++i) {
+    const bc4g_prepare_section& p = sections[i];
+    BC4G_REQUIRE(p.heads > 0 && p.dim > 0 && p.dim <= kMaxHead && p.half >= 0 && 2 * p.half <= p.dim,
+                 "heads_prepare: bad sizes heads=%d dim=%d (at most %d) half=%d", p.heads, p.dim, kMaxHead, p.half);
+    BC4G_REQUIRE(p.in && p.out && (p.half == 0 || p.table) && p.in_row >= static_cast<long>(p.heads) * p.dim &&
+                 (p.slot_map ? p.page_tokens > 0 : p.out_row >= static_cast<long>(p.heads) * p.dim) &&
+                 (p.in_dtype == kF32 || p.in_dtype == kBF16) && (p.out_dtype == kF32 || p.out_dtype == kBF16),
+                 "heads_prepare: a tensor is missing, a row is shorter than its heads, or a dtype is unknown");
+    all.s[i] = p;
+    heads += p.heads;
+  }
+  all.n = n_sections;
+  BC4G_REQUIRE(heads <= 65535, "heads_prepare: %ld heads are beyond the grid limit", heads);
+  if (n_rows == 0) return 0;
+  dim3 grid(n_rows, static_cast<unsigned>(heads));
+  heads_prepare_kernel<<<grid, kWave, 0, static_cast<hipStream_t>(stream)>>>(all);
+  return check_launch("heads_prepare");
+}
+
 extern "C" int bc4g_heads_prepare(const void* in, int in_dtype, long in_row, const float* bias, const float* norm_w, float eps,
                                   const float* table, int half, float factor, void* out, int out_dtype, long out_row,
                                   const int32_t* slot_map, int page_tokens, long page_stride, long head_stride,
                                   long token_stride, int n_rows, int heads, int dim, void* stream) {
-  BC4G_REQUIRE(n_rows >= 0 && heads > 0 && heads <= 65535 && dim > 0 && dim <= kMaxHead && half >= 0 && 2 * half <= dim,
-               "heads_prepare: bad sizes rows=%d heads=%d dim=%d (at most %d) half=%d", n_rows, heads, dim, kMaxHead, half);
-  BC4G_REQUIRE(in && out && (half == 0 || table) && in_row >= static_cast<long>(heads) * dim &&
-               (slot_map ? page_tokens > 0 : out_row >= static_cast<long>(heads) * dim) &&
-               (in_dtype == kF32 || in_dtype == kBF16) && (out_dtype == kF32 || out_dtype == kBF16),
-               "heads_prepare: a tensor is missing, a row is shorter than its heads, or a dtype is unknown");
-  if (n_rows == 0) return 0;
-  dim3 grid(n_rows, heads);
-  heads_prepare_kernel<<<grid, kWave, 0, static_cast<hipStream_t>(stream)>>>(
-      in, in_dtype, in_row, bias, norm_w, eps, table, half, factor, out, out_dtype, out_row, slot_map, page_tokens, page_stride,
-      head_stride, token_stride, dim);
-  return check_launch("heads_prepare");
+  const bc4g_prepare_section one{in, bias, norm_w, table, out, slot_map, in_row, out_row, page_stride, head_stride, token_stride,
+                                 in_dtype, out_dtype, half, page_tokens, heads, dim, eps, factor};
+  return bc4g_heads_prepare_many(&one, 1, n_rows, stream);
 }
 
 extern "C" int bc4g_heads_finish(const float* o, const float* w, float eps, float factor, const void* gate, int gate_dtype,

@@ -16,7 +16,7 @@ namespace bc4g {
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kMaxStreams = 8;
+constexpr int kMaxStreams = 16;
 
 int grid_for(long total) {
   const long g = (total + kBlock - 1) / kBlock;
@@ -46,8 +46,9 @@ __global__ void streams_read_kernel(const float* __restrict__ x, const int32_t* 
   }
 }
 
-// The write, and with next_out the next reader's input from the new copies.
-template <typename TO>
+// The write, and with next_out the next reader's input from the new copies.  NS: the most copies this instance holds in
+// registers (4, 8 or 16).
+template <typename TO, int NS>
 __global__ void streams_write_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ mix,
                                      const float* __restrict__ write, const float* __restrict__ next_read,
                                      const float* __restrict__ alpha, const float* __restrict__ g,
@@ -62,17 +63,17 @@ __global__ void streams_write_kernel(float* __restrict__ x, const float* __restr
     const int c = static_cast<int>(idx % hidden);
     const long r = idx / hidden;
     float* xr = x + r * n * hidden + c;
-    float old[kMaxStreams];
+    float old[NS];
 #pragma unroll
-    for (int s = 0; s < kMaxStreams; ++s) old[s] = s < n ? xr[static_cast<long>(s) * hidden] : 0.f;
+    for (int s = 0; s < NS; ++s) old[s] = s < n ? xr[static_cast<long>(s) * hidden] : 0.f;
     const float yv = y[idx];
     float u = 0.f;
 #pragma unroll
-    for (int t = 0; t < kMaxStreams; ++t) {
+    for (int t = 0; t < NS; ++t) {
       if (t >= n) break;
       float acc = 0.f;
 #pragma unroll
-      for (int s = 0; s < kMaxStreams; ++s)
+      for (int s = 0; s < NS; ++s)
         if (s < n) acc = fmaf(mix_s[s * n + t], old[s], acc);
       acc = fmaf(write_s[t], yv, acc);
       xr[static_cast<long>(t) * hidden] = acc;
@@ -125,13 +126,16 @@ extern "C" int bc4g_streams_write(float* x, const float* y, const float* mix, co
   if (n_rows == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const long total = static_cast<long>(n_rows) * hidden;
-  if (out_dtype == kF32)
-    streams_write_kernel<float><<<grid_for(total), kBlock, 0, s>>>(x, y, mix, write, next_read, alpha, g, b,
-                                                                   static_cast<float*>(next_out), total, n_streams, hidden);
-  else if (out_dtype == kBF16)
-    streams_write_kernel<bf16_t><<<grid_for(total), kBlock, 0, s>>>(x, y, mix, write, next_read, alpha, g, b,
-                                                                    static_cast<bf16_t*>(next_out), total, n_streams, hidden);
+#define BC4G_WRITE(TO, NS)                                                                                              \
+  streams_write_kernel<TO, NS><<<grid_for(total), kBlock, 0, s>>>(x, y, mix, write, next_read, alpha, g, b,              \
+                                                                  static_cast<TO*>(next_out), total, n_streams, hidden)
+#define BC4G_WRITE_N(TO)                                                                                                \
+  do { if (n_streams <= 4) BC4G_WRITE(TO, 4); else if (n_streams <= 8) BC4G_WRITE(TO, 8); else BC4G_WRITE(TO, 16); } while (0)
+  if (out_dtype == kF32) BC4G_WRITE_N(float);
+  else if (out_dtype == kBF16) BC4G_WRITE_N(bf16_t);
   else return fail("streams_write: unknown dtype %d", out_dtype);
+#undef BC4G_WRITE_N
+#undef BC4G_WRITE
   return check_launch("streams_write");
 }
 

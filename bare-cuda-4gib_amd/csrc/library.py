@@ -56,6 +56,7 @@ _SIGNATURES = {
     "bc4g_streams_fill": [_P, _P, _I, _I, _I, _P],
     "bc4g_rotary_table": [_P, _P, c_double, _P, _I, _I, _P],
     "bc4g_heads_prepare": [_P, _I, c_long, _P, _P, _F, _P, _I, _F, _P, _I, c_long, _P, _I, c_long, c_long, c_long, _I, _I, _I, _P],
+    "bc4g_heads_prepare_many": [_P, _I, _I, _P],
     "bc4g_heads_finish": [_P, _P, _F, _F, _P, _I, c_long, _I, _P, _I, _I, _I, _I, _P],
     "bc4g_decay_scan": [_P, _I, c_long, _F, _P, _I, c_long, _P, _I, c_long, _P, _P, _I, c_long, _P, _F, _P, _P, _P, _P, _P, _P, _P,
                         _I, _I, _I, _I, _I, _I, _P],

@@ -1401,7 +1401,7 @@ def attention_latent_work(ctx, heads: int, rank: int, rot: int, window: int, ele
 
 # ---- a residual stream in several copies, a pointwise norm, clamped gated units -----------------------------------------
 
-MAX_STREAMS = 8             # copies of the residual stream the kernels take
+MAX_STREAMS = 16            # copies of the residual stream the kernels take
 
 
 def _streams(what: str, x: torch.Tensor):
@@ -1510,13 +1510,23 @@ def rotary_table(positions: torch.Tensor, freqs: torch.Tensor, amplitude: float 
     return table
 
 
-def heads_prepare(x: torch.Tensor, heads: int, dim: int, out: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
+class _PrepareSection(ctypes.Structure):
+    """One section of heads_prepare_many, as the library's ``bc4g_prepare_section``."""
+    _fields_ = [("src", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("norm_w", ctypes.c_void_p), ("table", ctypes.c_void_p),
+                ("out", ctypes.c_void_p), ("slot_map", ctypes.c_void_p), ("in_row", ctypes.c_long), ("out_row", ctypes.c_long),
+                ("page_stride", ctypes.c_long), ("head_stride", ctypes.c_long), ("token_stride", ctypes.c_long),
+                ("in_dtype", ctypes.c_int), ("out_dtype", ctypes.c_int), ("half", ctypes.c_int), ("page_tokens", ctypes.c_int),
+                ("heads", ctypes.c_int), ("dim", ctypes.c_int), ("eps", ctypes.c_float), ("factor", ctypes.c_float)]
+
+
+def heads_section(x: torch.Tensor, heads: int, dim: int, out: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
                   norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0, table: Optional[torch.Tensor] = None,
-                  factor: float = 1.0, slot_map: Optional[torch.Tensor] = None, page_tokens: int = 0) -> torch.Tensor:
-    """Every head of x [T, heads * dim] (may be a part of wider rows): + bias, RMS norm over the head with
-    ``norm_weight`` [dim], rotation by ``table`` [T, half, 2] (element i with element i + half), times ``factor``.
-    ``out``: [T, heads, dim] (float32 or bfloat16), or with ``slot_map`` a cache [pages, heads, page_tokens, dim] whose
-    slot page * page_tokens + offset receives the row."""
+                  factor: float = 1.0, slot_map: Optional[torch.Tensor] = None, page_tokens: int = 0):
+    """One section for heads_prepare_many: every head of x [T, heads * dim] (may be a part of wider rows): + bias, RMS norm
+    over the head with ``norm_weight`` [dim], rotation by ``table`` [T, half, 2] (element i with element i + half), times
+    ``factor``.  ``out``: [T, heads, dim] (float32 or bfloat16), or with ``slot_map`` a cache
+    [pages, heads, page_tokens, dim] whose slot page * page_tokens + offset receives the row.  Checked here; the tensors
+    must live until the launch."""
     _dev("heads_prepare", bias, norm_weight, table, out, slot_map)
     in_row = _part_of_rows("heads_prepare", "x", x, heads * dim)
     t = x.shape[0]
@@ -1538,10 +1548,25 @@ def heads_prepare(x: torch.Tensor, heads: int, dim: int, out: torch.Tensor, *, b
             raise KernelError(f"heads_prepare: out must be [{t}, {heads}, {dim}], got {tuple(out.shape)}")
         page_stride = head_stride = token_stride = 0
         out_row = heads * dim
-    library.call("bc4g_heads_prepare", _ptr(x), _code(x, "heads_prepare"), in_row, _ptr(bias), _ptr(norm_weight), float(eps),
-                 _ptr(table), half, float(factor), _ptr(out), _code(out, "heads_prepare"), out_row, _ptr(slot_map), page_tokens,
-                 page_stride, head_stride, token_stride, t, heads, dim, _stream(),
-                 cost=lambda: (8.0 * t * heads * dim, t * heads * dim * (x.element_size() + out.element_size())))
+    section = _PrepareSection(_ptr(x), _ptr(bias), _ptr(norm_weight), _ptr(table), _ptr(out), _ptr(slot_map), in_row, out_row,
+                              page_stride, head_stride, token_stride, _code(x, "heads_prepare"), _code(out, "heads_prepare"), half,
+                              page_tokens, heads, dim, float(eps), float(factor))
+    return section, t, t * heads * dim, x.element_size() + out.element_size()
+
+
+def heads_prepare_many(sections) -> None:
+    """Up to four sections (heads_section) of the same step's rows in one launch: the queries, keys and values of an
+    attention layer, say."""
+    if not 1 <= len(sections) <= 4 or len({s[1] for s in sections}) != 1:
+        raise KernelError(f"heads_prepare: {len(sections)} sections (1 to 4) of {sorted({s[1] for s in sections})} rows")
+    array = (_PrepareSection * len(sections))(*[s[0] for s in sections])
+    library.call("bc4g_heads_prepare_many", ctypes.cast(array, ctypes.c_void_p), len(sections), sections[0][1], _stream(),
+                 cost=lambda: (8.0 * sum(s[2] for s in sections), sum(s[2] * s[3] for s in sections)))
+
+
+def heads_prepare(x: torch.Tensor, heads: int, dim: int, out: torch.Tensor, **how) -> torch.Tensor:
+    """One section alone (see heads_section); returns ``out``."""
+    heads_prepare_many([heads_section(x, heads, dim, out, **how)])
     return out
 
 

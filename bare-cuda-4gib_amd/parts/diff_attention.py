@@ -93,12 +93,14 @@ class DifferentialAttention(Part):
         q, k, v, g = x[:, :nq], x[:, nq:nq + nk], x[:, nq + nk:nq + nk + nv], x[:, nq + nk + nv:]
         table = self.position.table(ctx) if self.position is not None and hasattr(self.position, "table") else None
         q_maps = torch.empty((t, H * 2, d), dtype=torch.float32, device=x.device)
-        ops.heads_prepare(q, H * 2, d, q_maps, bias=self.q_b, norm_weight=self.q_norm, eps=self.eps, table=table)
+        # queries dense in float32, keys and values straight into their pages: one launch for the three
+        sections = [ops.heads_section(q, H * 2, d, q_maps, bias=self.q_b, norm_weight=self.q_norm, eps=self.eps, table=table)]
         if writes:
             slots = ctx.slot_maps[cache.group]
-            ops.heads_prepare(k, G * 2, d, cache.k, bias=self.k_b, norm_weight=self.k_norm, eps=self.eps, table=table,
-                              slot_map=slots, page_tokens=cache.page_tokens)
-            ops.heads_prepare(v, G, e, cache.v, bias=self.v_b, slot_map=slots, page_tokens=cache.page_tokens)
+            sections.append(ops.heads_section(k, G * 2, d, cache.k, bias=self.k_b, norm_weight=self.k_norm, eps=self.eps, table=table,
+                                              slot_map=slots, page_tokens=cache.page_tokens))
+            sections.append(ops.heads_section(v, G, e, cache.v, bias=self.v_b, slot_map=slots, page_tokens=cache.page_tokens))
+        ops.heads_prepare_many(sections)
         o = ops.attention_maps(q_maps.view(t, H, 2, d), cache.k, cache.v, ctx.block_tables[cache.group], ctx, self.act_dtype,
                                H, G, 2, d, e, self.window, self.keep_first, self.scale, lam=self.lam, normalize=True,
                                eps=self.eps, factor=1.0 - self.diff, gate=g, act=ops.ACT_SIGMOID)

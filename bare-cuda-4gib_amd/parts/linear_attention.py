@@ -90,8 +90,8 @@ class Retention(_DecayedState):
         q, k, v, g = x[:, :H * d], x[:, H * d:2 * H * d], x[:, 2 * H * d:2 * H * d + H * e], x[:, 2 * H * d + H * e:]
         table = self.position.table(ctx) if self.position is not None and hasattr(self.position, "table") else None
         qk = torch.empty((2, t, H, d), dtype=torch.float32, device=x.device)
-        ops.heads_prepare(q, H, d, qk[0], table=table)
-        ops.heads_prepare(k, H, d, qk[1], table=table, factor=d ** -0.5)
+        ops.heads_prepare_many([ops.heads_section(q, H, d, qk[0], table=table),
+                                ops.heads_section(k, H, d, qk[1], table=table, factor=d ** -0.5)])
         base, n_chunks = self._chunks(ctx)
         o = ops.decay_scan(qk[0].view(t, H * d), qk[1].view(t, H * d), v, cache.state, ctx, H, d, e, head_decay=self.head_decay,
                            chunk_base=base, n_chunks=n_chunks)

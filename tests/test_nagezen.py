@@ -72,7 +72,7 @@ def test_what_is_refused():
                    lambda c: c["layers"][1]["mixer"]["rot"].update(dims=14),        # more than a map has
                    lambda c: c["layers"][1]["mixer"]["rot"]["scaling"].pop("slow"),
                    lambda c: c["layers"][2]["mixer"].update(tau=0.0),
-                   lambda c: c.update(streams=9),
+                   lambda c: c.update(streams=17),
                    lambda c: c.pop("norm")):
         with pytest.raises(ConfigError):
             arch, cfg = _describe(broken(change))

@@ -245,7 +245,7 @@ def step_context(lengths, cached, slots):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("n", [1, 2, 5, 8])
+@pytest.mark.parametrize("n", [1, 2, 5, 8, 11, 16])
 def test_streams_are_read_written_and_filled(dtype, n):
     """The copies of the stream: the read with and without the norm, at chosen rows; the write from the OLD copies
     (a matrix far from symmetric, so that [from, to] the wrong way round shows), with the next read riding along."""
