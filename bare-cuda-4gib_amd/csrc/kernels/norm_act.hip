@@ -72,6 +72,33 @@ __global__ void clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ out
   }
 }
 
+// The same for bfloat16 and I a multiple of 8: a thread takes eight neighbouring outputs, in pieces of 16 bytes.
+__global__ void clamped_glu_pieces_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, float limit, float slope,
+                                          long pieces, int inter) {
+  const int per_row = inter / 8;
+  const long stride = static_cast<long>(blockDim.x) * gridDim.x;
+  for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < pieces; i += stride) {
+    const long r = i / per_row;
+    const int c = static_cast<int>(i - r * per_row) * 8;
+    const uint4 gv = *reinterpret_cast<const uint4*>(gu + r * 2 * inter + c);
+    const uint4 uv = *reinterpret_cast<const uint4*>(gu + r * 2 * inter + inter + c);
+    const unsigned gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
+    unsigned o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float res[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const float g = fminf(__uint_as_float(j ? gw[e] & 0xffff0000u : gw[e] << 16), limit);
+        const float u = fminf(fmaxf(__uint_as_float(j ? uw[e] & 0xffff0000u : uw[e] << 16), -limit), limit);
+        res[j] = g / (1.0f + expf(-slope * g)) * (u + 1.0f);
+      }
+      o[e] = static_cast<unsigned>(bf16_bits_from_float(res[0])) | (static_cast<unsigned>(bf16_bits_from_float(res[1])) << 16);
+    }
+    *reinterpret_cast<uint4*>(out + r * inter + c) = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+
 int grid_for(long total) {
   const long g = (total + kBlock - 1) / kBlock;
   return static_cast<int>(g < 1 ? 1 : (g > 65535 ? 65535 : g));
@@ -111,6 +138,8 @@ extern "C" int bc4g_clamped_glu(const void* gu, void* out, int dtype, float limi
   hipStream_t s = static_cast<hipStream_t>(stream);
   const long total = static_cast<long>(n_rows) * inter;
   if (dtype == kF32) clamped_glu_kernel<float><<<grid_for(total), kBlock, 0, s>>>(static_cast<const float*>(gu), static_cast<float*>(out), limit, slope, total, inter);
+  else if (dtype == kBF16 && inter % 8 == 0 && reinterpret_cast<uintptr_t>(gu) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0)
+    clamped_glu_pieces_kernel<<<grid_for(total / 8), kBlock, 0, s>>>(static_cast<const bf16_t*>(gu), static_cast<bf16_t*>(out), limit, slope, total / 8, inter);
   else if (dtype == kBF16) clamped_glu_kernel<bf16_t><<<grid_for(total), kBlock, 0, s>>>(static_cast<const bf16_t*>(gu), static_cast<bf16_t*>(out), limit, slope, total, inter);
   else return fail("clamped_glu: unknown dtype %d", dtype);
   return check_launch("clamped_glu");

@@ -246,12 +246,13 @@ def step_context(lengths, cached, slots):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("n", [1, 2, 5, 8, 11, 16])
-def test_streams_are_read_written_and_filled(dtype, n):
+@pytest.mark.parametrize("H", [37, 40])
+def test_streams_are_read_written_and_filled(dtype, n, H):
     """The copies of the stream: the read with and without the norm, at chosen rows; the write from the OLD copies
     (a matrix far from symmetric, so that [from, to] the wrong way round shows), with the next read riding along."""
     from bare_cuda_4gib_amd.csrc import ops
     torch.manual_seed(n)
-    T, H = 7, 37
+    T = 7
     x0 = torch.randn(T, H)
     x = ops.streams_fill(x0.to(DEV), n)
     assert torch.equal(x.cpu(), x0[:, None, :].expand(T, n, H))
@@ -280,15 +281,16 @@ def test_streams_are_read_written_and_filled(dtype, n):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_clamped_gated_unit(dtype):
+@pytest.mark.parametrize("inter", [53, 56])
+def test_clamped_gated_unit(dtype, inter):
     """Values on both sides of the limit in both branches: the gate is clamped from above only, the other branch on both
     sides, and one is added to it after the clamp."""
     from bare_cuda_4gib_amd.csrc import ops
     torch.manual_seed(3)
-    gu = (torch.randn(9, 2 * 53) * 3).to(dtype)
+    gu = (torch.randn(9, 2 * inter) * 3).to(dtype)
     for limit in (0.5, 2.5):
         got = ops.clamped_glu(gu.to(DEV), limit, 1.702).cpu().double()
-        want = plain.clamped_glu(gu[:, :53].double(), gu[:, 53:].double(), limit)
+        want = plain.clamped_glu(gu[:, :inter].double(), gu[:, inter:].double(), limit)
         tol = 1e-5 if dtype == torch.float32 else 1e-2
         assert torch.allclose(got, want, atol=tol, rtol=tol)
     assert float(plain.clamped_glu(torch.tensor([-9.0]), torch.tensor([0.0]), 2.5)) < -1e-6      # (no clamp below on the gate)
